@@ -1,0 +1,158 @@
+/*
+ * opencnn_amd — C ABI of the MI355X (gfx950) Winograd F(2x2,3x3) forward convolution.
+ *
+ * Plain C: pointers and sizes only.  Every device pointer is memory the CALLER
+ * allocated on the current HIP device; the library allocates nothing and keeps no
+ * state between calls except the stream selected with opencnn_set_stream().
+ * All entry points return a hipError_t value as int (0 == hipSuccess); launches are
+ * asynchronous on the selected stream, exactly like the reference, which returns
+ * cudaGetLastError() right after its two launches
+ * (src/convolutionForward_32x64x8.cu:274-283).
+ *
+ * Tensor layouts (row-major, last index fastest), as in the reference:
+ *   input   CHWN  [in_c][in_h][in_w][in_n]      src/openCNN_winograd.cu:149-150,230
+ *   filter  CRSK  [filt_c][3][3][filt_k]        src/openCNN_winograd.cu:235, src/FX_m2.cu:56-57
+ *   output  KHWN  [out_c][out_h][out_w][out_n]  src/store_and_transform_output_optSTS64.cuh:85-87
+ *   Ww      filt_c*16*filt_k floats of caller-owned scratch, overwritten by every call
+ *           (src/openCNN_winograd.cu:310-311).  Its CONTENT is the transformed filter
+ *           U = G g G^T in an MFMA-operand order private to this library; use
+ *           opencnn_filter_transform(..., OPENCNN_WW_REFERENCE) to obtain the reference's
+ *           [filt_c][16][filt_k] order (src/FX_m2.cu:58-59,84).
+ */
+#ifndef OPENCNN_AMD_H
+#define OPENCNN_AMD_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Layout of the transformed-filter buffer written by opencnn_filter_transform. */
+enum {
+  OPENCNN_WW_REFERENCE = 0, /* [filt_c][16][filt_k], position p = i*4+j (src/FX_m2.cu:84) */
+  OPENCNN_WW_MFMA = 1       /* [filt_k/32][filt_c/4][16][2][32][2]: what the fused kernel reads */
+};
+
+/* Layout of the 3x3 filters handed to the library. */
+enum {
+  OPENCNN_FILTER_CRSK = 0, /* what the reference's FX reads (src/FX_m2.cu:69) */
+  OPENCNN_FILTER_KCRS = 1  /* the cuDNN-side layout of the reference's bench (src/openCNN_winograd.cu:234) */
+};
+
+/* GEMM operand precision of the fused kernel (transforms and accumulation stay fp32). */
+enum { OPENCNN_F32 = 0, OPENCNN_F16 = 1, OPENCNN_BF16 = 2 };
+
+/*
+ * Replaces the reference's hidden set-up: the caller-side cudaMemcpyToSymbol uploads of
+ * the fragment-address tables (src/openCNN_winograd.cu:319-331).  This library has no
+ * such tables; the call checks that the current device is a gfx950 part and returns
+ * hipErrorInvalidDevice otherwise.  Calling it is optional.
+ */
+int opencnn_init(void);
+
+/*
+ * Drop-in for the reference's host dispatcher
+ *   cudaError_t convolutionForward(float *k, int in_h, int in_w, float *w, int out_h,
+ *       int out_w, int out_n, int out_c, float *C, float *Ww, const unsigned int n,
+ *       int tiles_dim, int in_n, int tile_size, int elems_dim, int in_c, int filt_k,
+ *       int filt_c, int filt_h, int filt_w, int alpha, int m)
+ * (src/openCNN_winograd.cu:204-219): same 22 arguments, same meaning, same layouts.
+ * Runs the filter transform and then the fused kernel, stream-ordered, on the stream
+ * set by opencnn_set_stream (default: the null stream, as in the reference).
+ *
+ * Unlike the reference, which mis-computes silently or returns an uninitialised value
+ * on shapes it does not support (src/openCNN_winograd.cu:212-218), unsupported
+ * arguments return hipErrorInvalidValue and launch nothing.  Supported: filt_h ==
+ * filt_w == 3, m == 2, alpha == tile_size == 4, in_n % 32 == 0, filt_k % 32 == 0,
+ * in_c % 8 == 0, filt_c == in_c, out_* consistent with pad 1 / stride 1, tiles_dim ==
+ * opencnn_tiles_dim(in_w), in_h == in_w, every tensor below 2^31 elements.
+ */
+int convolutionForward(float *k, int in_h, int in_w, float *w, int out_h, int out_w,
+                       int out_n, int out_c, float *C, float *Ww, const unsigned int n,
+                       int tiles_dim, int in_n, int tile_size, int elems_dim, int in_c,
+                       int filt_k, int filt_c, int filt_h, int filt_w, int alpha, int m);
+
+/*
+ * The reference's launcher behind the dispatcher, same arguments minus elems_dim
+ * (src/convolutionForward_32x64x8.cu:264-284).  Kept so code that binds the launcher
+ * directly keeps linking; the name's 32x64x8 is the reference's CUDA tile shape and
+ * says nothing about the tiling used here.
+ */
+int convolutionForward_32x64x8(float *k, int in_h, int in_w, float *w, int out_h,
+                               int out_w, int out_n, int out_c, float *C, float *Ww,
+                               const unsigned int n, int tiles_dim, int in_n,
+                               int tile_size, int in_c, int filt_k, int filt_c,
+                               int filt_h, int filt_w, int alpha, int m);
+
+/* tiles per image side, ceil(ceil((in_w+2)/2)-1): the caller-side computation at
+ * src/openCNN_winograd.cu:286-288. */
+int opencnn_tiles_dim(int in_w);
+
+/* Size in bytes of the Ww scratch: filt_k*filt_c*16*sizeof(float), the caller-side
+ * cudaMalloc at src/openCNN_winograd.cu:310-311. */
+size_t opencnn_workspace_bytes(int filt_c, int filt_k);
+
+/* Stream (a hipStream_t passed as void*) used by every later call from any thread;
+ * NULL selects the null stream, which is what the reference launches on
+ * (src/convolutionForward_32x64x8.cu:274,281). */
+int opencnn_set_stream(void *stream);
+
+/*
+ * The reference's FX kernel as a call of its own (src/FX_m2.cu:51-91, launched at
+ * src/convolutionForward_32x64x8.cu:274): U = G g G^T for every (c,k).
+ *   w              device, filt_c*9*filt_k floats in `filter_layout`
+ *   Ww             device, filt_c*16*filt_k floats, written in `ww_layout`
+ * OPENCNN_WW_REFERENCE output is bit-identical to the reference's arithmetic order
+ * (only additions and multiplications by 0.5).
+ */
+int opencnn_filter_transform(const float *w, float *Ww, int filt_k, int filt_c,
+                             int filter_layout, int ww_layout);
+
+/*
+ * The reference's Winograd_kernel as a call of its own
+ * (src/convolutionForward_32x64x8.cu:169-262, launched at :281): input transform,
+ * 16 batched GEMMs and output transform, reading a Ww that
+ * opencnn_filter_transform(..., OPENCNN_WW_MFMA) wrote earlier on the same stream.
+ * Lets a caller transform the filters once and reuse them, which the reference's
+ * dispatcher cannot (it re-runs FX on every call).  in_h and in_w may differ here.
+ */
+int opencnn_conv_forward_pretransformed(const float *in, const float *Ww, float *out,
+                                        int in_n, int in_c, int in_h, int in_w,
+                                        int filt_k);
+
+/*
+ * Bench support, the library-side twin of the reference's timing loop
+ * (src/openCNN_winograd.cu:426-444): `warmup` untimed calls, then `iters` back-to-back
+ * calls bracketed by HIP events on the selected stream.  Writes mean milliseconds per
+ * call of (a) filter transform + fused kernel, the quantity the reference reports,
+ * (b) the fused kernel alone, (c) the filter transform alone.  Synchronises the stream.
+ */
+int opencnn_time_forward(const float *in, const float *w, float *out, float *Ww,
+                         int in_n, int in_c, int in_h, int in_w, int filt_k, int warmup,
+                         int iters, float *ms_total, float *ms_main, float *ms_fx);
+
+/* Layout of a synthetic input written by opencnn_synth_input. */
+enum { OPENCNN_INPUT_CHWN = 0, OPENCNN_INPUT_NCHW = 1 };
+/* Distribution of a synthetic tensor: uniform on [p0,p1) or normal(mean p0, std p1). */
+enum { OPENCNN_DIST_UNIFORM = 0, OPENCNN_DIST_NORMAL = 1 };
+
+/*
+ * Seeded synthetic tensors in HOST memory (no GPU involved).  They stand in for the
+ * reference's unseeded curand fills and data_cpy transposes
+ * (src/openCNN_winograd.cu:127-153,221-238): element values depend only on
+ * (seed, logical NCHW / KCRS coordinate), so both layouts of a tensor hold the same
+ * numbers.  Return 0, or 1 on a bad argument.
+ */
+int opencnn_synth_input(float *dst, int n, int c, int h, int w, int layout,
+                        unsigned long long seed, int dist, double p0, double p1);
+int opencnn_synth_filter(float *dst, int k, int c, int layout, unsigned long long seed,
+                         int dist, double p0, double p1);
+
+/* Name of the last failing check in this thread ("" if none): a short static string. */
+const char *opencnn_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OPENCNN_AMD_H */

@@ -1,0 +1,213 @@
+"""ctypes binding of ``libopencnn_amd.so`` (the C ABI declared in ``include/opencnn_amd.h``).
+
+Device buffers are passed as ``torch`` CUDA(ROCm) tensors or raw integer addresses;
+torch is only the owner of device memory and streams here.  Every wrapper raises
+:class:`OpenCNNError` on a non-zero status.  Nothing in this module computes a
+convolution on the CPU: without the built library there is no product path.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional
+
+import numpy as np
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libopencnn_amd.so")
+
+# enum values of include/opencnn_amd.h
+WW_REFERENCE, WW_MFMA = 0, 1
+FILTER_CRSK, FILTER_KCRS = 0, 1
+INPUT_CHWN, INPUT_NCHW = 0, 1
+DIST_UNIFORM, DIST_NORMAL = 0, 1
+
+_c_int, _c_float_p, _c_void_p = ctypes.c_int, ctypes.POINTER(ctypes.c_float), ctypes.c_void_p
+
+# name -> (restype, argtypes); one entry per declaration in include/opencnn_amd.h
+EXPORTED_SYMBOLS = {
+    "opencnn_init": (_c_int, []),
+    "convolutionForward": (
+        _c_int,
+        [_c_void_p, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p,
+         _c_void_p, ctypes.c_uint, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+         _c_int, _c_int, _c_int, _c_int],
+    ),
+    "convolutionForward_32x64x8": (
+        _c_int,
+        [_c_void_p, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p,
+         _c_void_p, ctypes.c_uint, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+         _c_int, _c_int, _c_int],
+    ),
+    "opencnn_tiles_dim": (_c_int, [_c_int]),
+    "opencnn_workspace_bytes": (ctypes.c_size_t, [_c_int, _c_int]),
+    "opencnn_set_stream": (_c_int, [_c_void_p]),
+    "opencnn_filter_transform": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int]),
+    "opencnn_conv_forward_pretransformed": (
+        _c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int]),
+    "opencnn_time_forward": (
+        _c_int,
+        [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
+         _c_int, _c_int, _c_float_p, _c_float_p, _c_float_p],
+    ),
+    "opencnn_synth_input": (
+        _c_int,
+        [_c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, ctypes.c_ulonglong, _c_int,
+         ctypes.c_double, ctypes.c_double],
+    ),
+    "opencnn_synth_filter": (
+        _c_int,
+        [_c_void_p, _c_int, _c_int, _c_int, ctypes.c_ulonglong, _c_int, ctypes.c_double,
+         ctypes.c_double],
+    ),
+    "opencnn_last_error": (ctypes.c_char_p, []),
+}
+
+
+class OpenCNNError(RuntimeError):
+    """A C-ABI call returned a non-zero hipError_t."""
+
+    def __init__(self, func: str, status: int, detail: str = ""):
+        self.func, self.status, self.detail = func, status, detail
+        msg = f"{func} failed with hipError_t {status}"
+        if detail:
+            msg += f" (failed check: {detail})"
+        super().__init__(msg)
+
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def load_library(path: str = LIB_PATH) -> ctypes.CDLL:
+    """Load the built HIP library; raises if it has not been built (no fallback)."""
+    global _lib
+    if _lib is not None and path == LIB_PATH:
+        return _lib
+    if not os.path.exists(path):
+        raise ImportError(
+            f"{path} is missing: build it with `make -C opencnn_amd/csrc` "
+            "(or __graft_entry__.build()); opencnn_amd has no non-HIP path")
+    handle = ctypes.CDLL(path)
+    for name, (restype, argtypes) in EXPORTED_SYMBOLS.items():
+        fn = getattr(handle, name)  # AttributeError if the symbol is not exported
+        fn.restype, fn.argtypes = restype, argtypes
+    if path == LIB_PATH:
+        _lib = handle
+    return handle
+
+
+def lib() -> ctypes.CDLL:
+    return load_library()
+
+
+def _ptr(buf) -> int:
+    """Address of a torch tensor / numpy array / raw int."""
+    if isinstance(buf, int):
+        return buf
+    if isinstance(buf, np.ndarray):
+        if not buf.flags["C_CONTIGUOUS"]:
+            raise ValueError("numpy buffer must be C-contiguous")
+        return buf.ctypes.data
+    if hasattr(buf, "data_ptr"):
+        if not buf.is_contiguous():
+            raise ValueError("tensor must be contiguous")
+        return buf.data_ptr()
+    raise TypeError(f"cannot take the address of {type(buf)!r}")
+
+
+def _dev_f32(buf, what: str) -> int:
+    if hasattr(buf, "is_cuda"):
+        import torch
+
+        if not buf.is_cuda:
+            raise ValueError(f"{what} must live in device memory")
+        if buf.dtype != torch.float32:
+            raise ValueError(f"{what} must be float32")
+    return _ptr(buf)
+
+
+def _check(func: str, status: int) -> None:
+    if status != 0:
+        detail = lib().opencnn_last_error().decode() if status == 1 else ""
+        raise OpenCNNError(func, status, detail)
+
+
+def init() -> None:
+    _check("opencnn_init", lib().opencnn_init())
+
+
+def tiles_dim(in_w: int) -> int:
+    return lib().opencnn_tiles_dim(in_w)
+
+
+def workspace_bytes(filt_c: int, filt_k: int) -> int:
+    return lib().opencnn_workspace_bytes(filt_c, filt_k)
+
+
+def set_stream(stream) -> None:
+    """Select the stream of later calls: a torch.cuda.Stream, a raw handle or None."""
+    handle = 0 if stream is None else getattr(stream, "cuda_stream", stream)
+    _check("opencnn_set_stream", lib().opencnn_set_stream(handle))
+
+
+def convolutionForward(k, in_h, in_w, w, out_h, out_w, out_n, out_c, C, Ww, n, tiles_dim,
+                       in_n, tile_size, elems_dim, in_c, filt_k, filt_c, filt_h, filt_w,
+                       alpha, m) -> None:
+    """The reference's dispatcher, argument for argument (src/openCNN_winograd.cu:204-209):
+    ``k`` CHWN input, ``w`` CRSK filters, ``C`` KHWN output, ``Ww`` workspace."""
+    _check("convolutionForward", lib().convolutionForward(
+        _dev_f32(k, "input"), in_h, in_w, _dev_f32(w, "filter"), out_h, out_w, out_n, out_c,
+        _dev_f32(C, "output"), _dev_f32(Ww, "workspace"), n, tiles_dim, in_n, tile_size,
+        elems_dim, in_c, filt_k, filt_c, filt_h, filt_w, alpha, m))
+
+
+def filter_transform(w, Ww, filt_k, filt_c, filter_layout=FILTER_CRSK,
+                     ww_layout=WW_REFERENCE) -> None:
+    _check("opencnn_filter_transform", lib().opencnn_filter_transform(
+        _dev_f32(w, "filter"), _dev_f32(Ww, "workspace"), filt_k, filt_c, filter_layout,
+        ww_layout))
+
+
+def conv_forward_pretransformed(x, Ww, y, in_n, in_c, in_h, in_w, filt_k) -> None:
+    _check("opencnn_conv_forward_pretransformed", lib().opencnn_conv_forward_pretransformed(
+        _dev_f32(x, "input"), _dev_f32(Ww, "workspace"), _dev_f32(y, "output"), in_n, in_c,
+        in_h, in_w, filt_k))
+
+
+def time_forward(x, w, y, Ww, in_n, in_c, in_h, in_w, filt_k, warmup=1, iters=100):
+    """Mean ms per call: (filter transform + fused kernel, fused kernel, filter transform)."""
+    t = [ctypes.c_float(0.0) for _ in range(3)]
+    _check("opencnn_time_forward", lib().opencnn_time_forward(
+        _dev_f32(x, "input"), _dev_f32(w, "filter"), _dev_f32(y, "output"),
+        _dev_f32(Ww, "workspace"), in_n, in_c, in_h, in_w, filt_k, warmup, iters,
+        ctypes.byref(t[0]), ctypes.byref(t[1]), ctypes.byref(t[2])))
+    return t[0].value, t[1].value, t[2].value
+
+
+def synth_input(n, c, h, w, seed, layout=INPUT_CHWN, dist=DIST_UNIFORM, p0=-1.0, p1=1.0):
+    """Seeded host tensor, shape (c,h,w,n) for CHWN or (n,c,h,w) for NCHW."""
+    shape = (c, h, w, n) if layout == INPUT_CHWN else (n, c, h, w)
+    out = np.empty(shape, dtype=np.float32)
+    _check("opencnn_synth_input", lib().opencnn_synth_input(
+        out.ctypes.data, n, c, h, w, layout, seed, dist, p0, p1))
+    return out
+
+
+def synth_filter(k, c, seed, layout=FILTER_CRSK, dist=DIST_NORMAL, p0=0.0, p1=None):
+    """Seeded host filters, shape (c,3,3,k) for CRSK or (k,c,3,3) for KCRS.
+    Default: He-init normal(0, sqrt(2/(9c)))."""
+    if p1 is None:
+        p1 = float(np.sqrt(2.0 / (9.0 * c)))
+    shape = (c, 3, 3, k) if layout == FILTER_CRSK else (k, c, 3, 3)
+    out = np.empty(shape, dtype=np.float32)
+    _check("opencnn_synth_filter", lib().opencnn_synth_filter(
+        out.ctypes.data, k, c, layout, seed, dist, p0, p1))
+    return out
+
+
+def unswizzle_ww(ww_mfma: np.ndarray, filt_c: int, filt_k: int) -> np.ndarray:
+    """Reorder a host copy of an OPENCNN_WW_MFMA buffer ([k/32][c/4][16][2][32][2]) into the
+    reference's [c][16][k] order (src/FX_m2.cu:84).  Pure permutation, no arithmetic."""
+    a = np.asarray(ww_mfma, dtype=np.float32).reshape(filt_k // 32, filt_c // 4, 16, 2, 32, 2)
+    # axes: kg, q, p, h, k32, s ; c = 4q + 2s + h ; k = 32kg + k32
+    a = a.transpose(1, 5, 3, 2, 0, 4)  # q, s, h, p, kg, k32
+    return np.ascontiguousarray(a).reshape(filt_c, 16, filt_k)

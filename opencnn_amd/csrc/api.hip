@@ -1,0 +1,217 @@
+// C ABI of opencnn_amd: argument validation and kernel launches.
+// Host-side counterpart of the reference's dispatcher and launcher
+// (src/openCNN_winograd.cu:204-219, src/convolutionForward_32x64x8.cu:264-284).
+#include "../../include/opencnn_amd.h"
+
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cmath>
+#include <cstring>
+
+#include "conv_kernel_f32.hpp"
+#include "fx_kernels.hpp"
+
+namespace {
+
+std::atomic<hipStream_t> g_stream{nullptr};
+thread_local const char* t_last_error = "";
+
+int fail(const char* what) {
+  t_last_error = what;
+  return (int)hipErrorInvalidValue;
+}
+
+#define REQUIRE(cond) \
+  do {                \
+    if (!(cond)) return fail(#cond); \
+  } while (0)
+
+constexpr long long kMaxElems = (1LL << 31) - 1;
+
+int check_filter_shape(int filt_k, int filt_c) {
+  REQUIRE(filt_k > 0 && filt_c > 0);
+  REQUIRE(filt_k % 32 == 0);
+  REQUIRE(filt_c % 8 == 0);
+  REQUIRE((long long)filt_k * filt_c * 16 <= kMaxElems / 4);  // Ww byte offsets stay below 2^31
+  return 0;
+}
+
+int check_conv_shape(int in_n, int in_c, int in_h, int in_w, int filt_k) {
+  REQUIRE(in_n > 0 && in_c > 0 && in_h > 0 && in_w > 0);
+  REQUIRE(in_n % 32 == 0);
+  if (int e = check_filter_shape(filt_k, in_c)) return e;
+  REQUIRE((long long)in_n * in_c * in_h * in_w <= kMaxElems);
+  REQUIRE((long long)in_n * filt_k * in_h * in_w <= kMaxElems);
+  REQUIRE((long long)in_n * in_h * in_w * 2 * 4 <= kMaxElems);  // two-channel slab in bytes
+  return 0;
+}
+
+int launch_fx(const float* w, float* Ww, int filt_k, int filt_c, int filter_layout,
+              int ww_layout, hipStream_t st) {
+  REQUIRE(w != nullptr && Ww != nullptr);
+  REQUIRE(filter_layout == OPENCNN_FILTER_CRSK || filter_layout == OPENCNN_FILTER_KCRS);
+  REQUIRE(ww_layout == OPENCNN_WW_REFERENCE || ww_layout == OPENCNN_WW_MFMA);
+  if (int e = check_filter_shape(filt_k, filt_c)) return e;
+  const bool kcrs = filter_layout == OPENCNN_FILTER_KCRS;
+  if (ww_layout == OPENCNN_WW_REFERENCE) {
+    dim3 grid((filt_k + 255) / 256, filt_c), block(256);
+    if (kcrs)
+      opencnn::fx_reference_layout<true><<<grid, block, 0, st>>>(w, Ww, filt_k, filt_c);
+    else
+      opencnn::fx_reference_layout<false><<<grid, block, 0, st>>>(w, Ww, filt_k, filt_c);
+  } else {
+    dim3 grid((filt_k + 127) / 128, filt_c / 4), block(256);
+    if (kcrs)
+      opencnn::fx_mfma_layout<true><<<grid, block, 0, st>>>(w, Ww, filt_k, filt_c);
+    else
+      opencnn::fx_mfma_layout<false><<<grid, block, 0, st>>>(w, Ww, filt_k, filt_c);
+  }
+  return (int)hipGetLastError();
+}
+
+int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c, int in_h,
+                int in_w, int filt_k, hipStream_t st) {
+  REQUIRE(in != nullptr && Ww != nullptr && out != nullptr);
+  if (int e = check_conv_shape(in_n, in_c, in_h, in_w, filt_k)) return e;
+  opencnn::ConvArgs a;
+  a.x = in;
+  a.usw = Ww;
+  a.y = out;
+  a.N = in_n;
+  a.C = in_c;
+  a.H = in_h;
+  a.W = in_w;
+  a.K = filt_k;
+  a.tiles_h = (in_h + 1) / 2;
+  a.tiles_w = (in_w + 1) / 2;
+  a.ngroups = in_n / 32;
+  a.colgroups = a.tiles_h * a.tiles_w * a.ngroups;
+  a.kgroups = filt_k / 32;
+  const long long colblocks = (a.colgroups + 3) / 4;
+  const long long nblocks = colblocks * a.kgroups;
+  REQUIRE(nblocks <= kMaxElems / 8);
+  a.nblocks = (int)nblocks;
+  const int per_xcd = (a.nblocks + 7) / 8;
+  dim3 grid(per_xcd * 8), block(256);
+  opencnn::wino_f32_fused<2><<<grid, block, 0, st>>>(a);
+  return (int)hipGetLastError();
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* opencnn_last_error(void) { return t_last_error; }
+
+int opencnn_init(void) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  hipDeviceProp_t prop;
+  e = hipGetDeviceProperties(&prop, dev);
+  if (e != hipSuccess) return (int)e;
+  if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+    t_last_error = "device is not gfx950";
+    return (int)hipErrorInvalidDevice;
+  }
+  return 0;
+}
+
+int opencnn_tiles_dim(int in_w) {
+  return (int)std::ceil(std::ceil((double)(in_w + 2) / 2.0) - 1.0);
+}
+
+size_t opencnn_workspace_bytes(int filt_c, int filt_k) {
+  if (filt_c <= 0 || filt_k <= 0) return 0;
+  return (size_t)filt_c * (size_t)filt_k * 16 * sizeof(float);
+}
+
+int opencnn_set_stream(void* stream) {
+  g_stream.store(static_cast<hipStream_t>(stream));
+  return 0;
+}
+
+int opencnn_filter_transform(const float* w, float* Ww, int filt_k, int filt_c,
+                             int filter_layout, int ww_layout) {
+  return launch_fx(w, Ww, filt_k, filt_c, filter_layout, ww_layout, g_stream.load());
+}
+
+int opencnn_conv_forward_pretransformed(const float* in, const float* Ww, float* out, int in_n,
+                                        int in_c, int in_h, int in_w, int filt_k) {
+  return launch_main(in, Ww, out, in_n, in_c, in_h, in_w, filt_k, g_stream.load());
+}
+
+int convolutionForward_32x64x8(float* k, int in_h, int in_w, float* w, int out_h, int out_w,
+                               int out_n, int out_c, float* C, float* Ww, const unsigned int n,
+                               int tiles_dim, int in_n, int tile_size, int in_c, int filt_k,
+                               int filt_c, int filt_h, int filt_w, int alpha, int m) {
+  (void)n;  // out_c*out_n*out_h*out_w in the reference's bench; unused there too
+  REQUIRE(k != nullptr && w != nullptr && C != nullptr && Ww != nullptr);
+  REQUIRE(filt_h == 3 && filt_w == 3);
+  REQUIRE(m == 2);
+  REQUIRE(alpha == 4 && tile_size == 4);
+  REQUIRE(in_h == in_w);  // the reference's masks and tiles_dim only model square images
+  REQUIRE(filt_c == in_c);
+  REQUIRE(out_h == in_h && out_w == in_w);  // pad 1, stride 1
+  REQUIRE(out_n == in_n && out_c == filt_k);
+  REQUIRE(tiles_dim == opencnn_tiles_dim(in_w));
+  if (int e = check_conv_shape(in_n, in_c, in_h, in_w, filt_k)) return e;
+  hipStream_t st = g_stream.load();
+  if (int e = launch_fx(w, Ww, filt_k, filt_c, OPENCNN_FILTER_CRSK, OPENCNN_WW_MFMA, st)) return e;
+  return launch_main(k, Ww, C, in_n, in_c, in_h, in_w, filt_k, st);
+}
+
+int convolutionForward(float* k, int in_h, int in_w, float* w, int out_h, int out_w, int out_n,
+                       int out_c, float* C, float* Ww, const unsigned int n, int tiles_dim,
+                       int in_n, int tile_size, int elems_dim, int in_c, int filt_k, int filt_c,
+                       int filt_h, int filt_w, int alpha, int m) {
+  (void)elems_dim;  // tiles_dim*4 in the reference's bench; unused there too
+  return convolutionForward_32x64x8(k, in_h, in_w, w, out_h, out_w, out_n, out_c, C, Ww, n,
+                                    tiles_dim, in_n, tile_size, in_c, filt_k, filt_c, filt_h,
+                                    filt_w, alpha, m);
+}
+
+int opencnn_time_forward(const float* in, const float* w, float* out, float* Ww, int in_n,
+                         int in_c, int in_h, int in_w, int filt_k, int warmup, int iters,
+                         float* ms_total, float* ms_main, float* ms_fx) {
+  REQUIRE(iters > 0 && warmup >= 0);
+  REQUIRE(in != nullptr && w != nullptr && out != nullptr && Ww != nullptr);
+  if (int e = check_conv_shape(in_n, in_c, in_h, in_w, filt_k)) return e;
+  hipStream_t st = g_stream.load();
+  hipEvent_t ev[2];
+  hipError_t he;
+  if ((he = hipEventCreate(&ev[0])) != hipSuccess) return (int)he;
+  if ((he = hipEventCreate(&ev[1])) != hipSuccess) {
+    (void)hipEventDestroy(ev[0]);
+    return (int)he;
+  }
+  int rc = 0;
+  auto fx = [&]() { return launch_fx(w, Ww, filt_k, in_c, OPENCNN_FILTER_CRSK, OPENCNN_WW_MFMA, st); };
+  auto maink = [&]() { return launch_main(in, Ww, out, in_n, in_c, in_h, in_w, filt_k, st); };
+  auto timed = [&](int mode, float* ms_out) {
+    // mode 0: fx + main, 1: main only, 2: fx only
+    for (int i = 0; i < warmup + iters && rc == 0; ++i) {
+      if (i == warmup) {
+        if ((he = hipStreamSynchronize(st)) != hipSuccess) { rc = (int)he; break; }
+        if ((he = hipEventRecord(ev[0], st)) != hipSuccess) { rc = (int)he; break; }
+      }
+      if (mode != 1) rc = fx();
+      if (rc == 0 && mode != 2) rc = maink();
+    }
+    if (rc != 0) return;
+    if ((he = hipEventRecord(ev[1], st)) != hipSuccess) { rc = (int)he; return; }
+    if ((he = hipEventSynchronize(ev[1])) != hipSuccess) { rc = (int)he; return; }
+    float ms = 0.f;
+    if ((he = hipEventElapsedTime(&ms, ev[0], ev[1])) != hipSuccess) { rc = (int)he; return; }
+    if (ms_out) *ms_out = ms / (float)iters;
+  };
+  if (ms_total) timed(0, ms_total);
+  if (rc == 0 && ms_fx) timed(2, ms_fx);
+  if (rc == 0 && ms_main) timed(1, ms_main);  // last: leaves Ww valid for the final output
+  (void)hipEventDestroy(ev[0]);
+  (void)hipEventDestroy(ev[1]);
+  return rc;
+}
+
+}  // extern "C"

@@ -1,0 +1,208 @@
+// Fused Winograd F(2x2,3x3) forward convolution, fp32 operands on fp32 MFMA, gfx950.
+//
+// Replaces the reference's Winograd_kernel and its helpers
+// (src/convolutionForward_32x64x8.cu:53-262, src/outer_product_suffle.cuh,
+// src/store_and_transform_output_optSTS64.cuh).  Same mathematics, different machine
+// mapping:
+//
+//  * GEMM view.  For each of the 16 Winograd positions p:
+//        M[p][k][(tile,n)] = sum_c U[p][k][c] * V[p][c][(tile,n)]
+//    k sits on the MFMA row side (A operand = transformed filter U), the batch index n
+//    on the column side (B operand = transformed input V).  One wave owns a
+//    32 k x 32 n tile of ONE spatial tile for ALL 16 positions: 16 accumulators of
+//    v_mfma_f32_32x32x2_f32 = 256 accumulator registers, one wave per SIMD.
+//  * Input path.  Lane (h, n) (h = lane/32, n = lane%32) loads the 4x4 patch of channel
+//    c0+h for batch element n0+n straight from CHWN memory: every load instruction is two
+//    fully used 128-byte rows.  The patch is transformed (B^T d B, 32 add/sub) in
+//    registers and IS the B operand of the MFMA: the transformed input never visits LDS.
+//    Zero padding is implicit: out-of-image patch elements use a buffer offset beyond
+//    num_records, for which buffer loads return 0 without touching memory
+//    (the reference's bit masks, src/convolutionForward_32x64x8.cu:179-183).
+//  * Output path.  Because a lane holds all 16 positions of its (k, n) elements, the
+//    output transform A^T M A is element-wise across accumulators; the reference's four
+//    rounds of shared-memory transposition
+//    (src/store_and_transform_output_optSTS64.cuh:97-127) have no counterpart.  In the
+//    MFMA D layout lanes 0-31 of an accumulator register are 32 consecutive n of one k,
+//    so each store instruction writes two complete 128-byte rows of KHWN.
+//  * Reduction order: channels ascending, two per MFMA step, fp32 accumulate
+//    (the reference: one FMA per channel, ascending, src/convolutionForward_32x64x8.cu:210-257).
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace opencnn {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+
+struct ConvArgs {
+  const float* x;    // CHWN
+  const float* usw;  // transformed filter, MFMA operand order (see fx_mfma_layout)
+  float* y;          // KHWN
+  int N, C, H, W, K;
+  int tiles_h, tiles_w;  // 2x2 output tiles per image column / row
+  int ngroups;           // N / 32
+  int colgroups;         // tiles_h * tiles_w * ngroups   (wave-level column tiles)
+  int kgroups;           // K / 32
+  int nblocks;           // ceil(colgroups / 4) * kgroups (4 waves = 4 column tiles per block)
+};
+
+// V = B^T d B, columns first then rows (src/convolutionForward_32x64x8.cu:59-80).
+__device__ __forceinline__ void input_transform(const float (&d)[16], float (&v)[16]) {
+  float t[16];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    t[0 + j] = d[0 + j] - d[8 + j];
+    t[4 + j] = d[4 + j] + d[8 + j];
+    t[8 + j] = d[8 + j] - d[4 + j];
+    t[12 + j] = d[4 + j] - d[12 + j];
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[i * 4 + 0] = t[i * 4 + 0] - t[i * 4 + 2];
+    v[i * 4 + 1] = t[i * 4 + 1] + t[i * 4 + 2];
+    v[i * 4 + 2] = t[i * 4 + 2] - t[i * 4 + 1];
+    v[i * 4 + 3] = t[i * 4 + 1] - t[i * 4 + 3];
+  }
+}
+
+// Y = A^T m A (src/store_and_transform_output_optSTS64.cuh:29-51), m[i*4+j] -> o[a*2+b].
+__device__ __forceinline__ void output_transform(const float (&m)[16], float (&o)[4]) {
+  float a[8];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    a[j] = (m[j] + m[4 + j]) + m[8 + j];
+    a[4 + j] = (m[4 + j] - m[8 + j]) - m[12 + j];
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    o[i * 2 + 0] = (a[i * 4 + 0] + a[i * 4 + 1]) + a[i * 4 + 2];
+    o[i * 2 + 1] = (a[i * 4 + 1] - a[i * 4 + 2]) - a[i * 4 + 3];
+  }
+}
+
+constexpr int kBufferFlags = 0x00020000;  // raw buffer, 32-bit data format (gfx9 family)
+constexpr int kOutOfRange = (int)0x80000000;  // voffset no num_records can reach
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, kBufferFlags);
+}
+
+// NBUF = number of 4x4 patches a lane keeps in flight ahead of the MFMA step that uses them.
+template <int NBUF>
+__global__ void __launch_bounds__(256) wino_f32_fused(ConvArgs a) {
+  static_assert(NBUF == 1 || NBUF == 2 || NBUF == 4, "NBUF must divide 4");
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+
+  // Workgroups are dealt round-robin to the 8 XCDs (one L2 each).  Give every XCD a
+  // contiguous range of logical blocks so that blocks sharing input columns (same
+  // column block, different k group) and filters (same k group) meet in one L2.
+  const int per_xcd = gridDim.x >> 3;
+  const int L = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (L >= a.nblocks) return;
+  const int kg = L % a.kgroups;
+  const int cg = (L / a.kgroups) * 4 + wave;
+  if (cg >= a.colgroups) return;  // wave-uniform; the kernel has no barriers
+
+  const int tile = cg / a.ngroups, ng = cg - tile * a.ngroups;
+  const int ty = tile / a.tiles_w, tx = tile - ty * a.tiles_w;
+  const int hsel = lane >> 5, nl = lane & 31;
+  const int HW = a.H * a.W;
+  const size_t HWN = (size_t)HW * a.N;
+
+  // Byte offset of patch element (i,j) inside a two-channel slab of x, or kOutOfRange.
+  int voff[16];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int hh = 2 * ty - 1 + i, ww = 2 * tx - 1 + j;
+      const bool ok = hh >= 0 && hh < a.H && ww >= 0 && ww < a.W;
+      voff[i * 4 + j] =
+          ok ? (int)(((size_t)hsel * HW + (size_t)hh * a.W + ww) * a.N + ng * 32 + nl) * 4
+             : kOutOfRange;
+    }
+  }
+  const unsigned slab_bytes = (unsigned)(2 * HWN * sizeof(float));
+  const int S = a.C >> 1;  // MFMA steps (two channels each)
+  const int Q = a.C >> 2;  // filter quads (two steps each)
+
+  auto load_patch = [&](float (&d)[16], int step) {
+    const int st = step < S ? step : S - 1;  // past the end: reload the last slab, unused
+    __amdgpu_buffer_rsrc_t r = make_rsrc(a.x + (size_t)st * 2 * HWN, slab_bytes);
+#pragma unroll
+    for (int e = 0; e < 16; ++e)
+      d[e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff[e], 0, 0));
+  };
+
+  const __amdgpu_buffer_rsrc_t ru =
+      make_rsrc(a.usw, (unsigned)((size_t)a.C * 16 * a.K * sizeof(float)));
+  const int uoff = lane * 8;
+  auto load_u = [&](v2f (&u)[16], int quad) {
+    const int qd = quad < Q ? quad : Q - 1;
+    const int soff = (kg * Q + qd) * (16 * 64 * 8);
+#pragma unroll
+    for (int p = 0; p < 16; ++p)
+      u[p] = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(ru, uoff + p * 512, soff, 0));
+  };
+
+  v16f acc[16];
+#pragma unroll
+  for (int p = 0; p < 16; ++p)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[p][r] = 0.0f;
+
+  v2f u[2][16];
+  float d[NBUF][16];
+  float v[2][16];
+
+  // prologue
+  load_u(u[0], 0);
+  {
+    float d0[16];
+    load_patch(d0, 0);
+#pragma unroll
+    for (int m = 1; m <= NBUF; ++m) load_patch(d[m % NBUF], m);
+    input_transform(d0, v[0]);
+  }
+
+  const int octs = a.C >> 3;
+  for (int oct = 0; oct < octs; ++oct) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int t = oct * 4 + s;
+      if (s == 0) load_u(u[1], 2 * oct + 1);
+      if (s == 2) load_u(u[0], 2 * oct + 2);
+      // transform the next step's patch while this step's MFMAs run
+      input_transform(d[(s + 1) % NBUF], v[(s + 1) & 1]);
+      load_patch(d[(s + 1) % NBUF], t + 1 + NBUF);
+#pragma unroll
+      for (int p = 0; p < 16; ++p)
+        acc[p] = __builtin_amdgcn_mfma_f32_32x32x2f32(u[s >> 1][p][s & 1], v[s & 1][p], acc[p], 0, 0, 0);
+    }
+  }
+
+  // Epilogue: accumulator register r of lane (hsel, nl) is row k = 8*(r/4) + 4*hsel + r%4,
+  // column n = nl of the 32x32 tile.
+  const bool row1 = 2 * ty + 1 < a.H;  // odd H: last tile row keeps only a = 0
+  const bool col1 = 2 * tx + 1 < a.W;  // odd W: last tile column keeps only b = 0
+  float* ybase = a.y + ((size_t)(2 * ty) * a.W + 2 * tx) * a.N + ng * 32 + nl;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    float m[16], o[4];
+#pragma unroll
+    for (int p = 0; p < 16; ++p) m[p] = acc[p][r];
+    output_transform(m, o);
+    const int k = kg * 32 + 8 * (r >> 2) + 4 * hsel + (r & 3);
+    float* yk = ybase + (size_t)k * HWN;
+    yk[0] = o[0];
+    if (col1) yk[a.N] = o[1];
+    if (row1) {
+      yk[(size_t)a.W * a.N] = o[2];
+      if (col1) yk[(size_t)a.W * a.N + a.N] = o[3];
+    }
+  }
+}
+
+}  // namespace opencnn

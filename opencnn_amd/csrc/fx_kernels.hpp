@@ -1,0 +1,89 @@
+// Filter transform U = G g G^T for Winograd F(2x2,3x3), gfx950.
+//
+// Replaces the reference's FX kernel (src/FX_m2.cu:51-91).  Arithmetic order follows
+// src/FX_m2.cu:23-47 exactly (rows: (g0+g2)+-g1 then x0.5; same along columns), so the
+// OPENCNN_WW_REFERENCE output is bit-identical to the reference's.
+//
+// HBM-bound streaming kernel: 9 floats in, 16 floats out per (c,k).
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace opencnn {
+
+// One 3x3 filter g[r*3+s] -> U[i*4+j].
+__device__ __forceinline__ void fx_one(const float (&g)[9], float (&U)[16]) {
+  float t[12];
+#pragma unroll
+  for (int s = 0; s < 3; ++s) {
+    t[0 * 3 + s] = g[s];
+    t[1 * 3 + s] = 0.5f * ((g[s] + g[6 + s]) + g[3 + s]);
+    t[2 * 3 + s] = 0.5f * ((g[s] + g[6 + s]) - g[3 + s]);
+    t[3 * 3 + s] = g[6 + s];
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    U[i * 4 + 0] = t[i * 3 + 0];
+    U[i * 4 + 1] = 0.5f * ((t[i * 3 + 0] + t[i * 3 + 2]) + t[i * 3 + 1]);
+    U[i * 4 + 2] = 0.5f * ((t[i * 3 + 0] + t[i * 3 + 2]) - t[i * 3 + 1]);
+    U[i * 4 + 3] = t[i * 3 + 2];
+  }
+}
+
+// Read one filter.  CRSK: w[(c*9+i)*K + k] (k contiguous across lanes).
+// KCRS: w[(k*C+c)*9 + i].
+template <bool KCRS>
+__device__ __forceinline__ void load_filter(const float* __restrict__ w, int c, int k, int C,
+                                            int K, float (&g)[9]) {
+  if (KCRS) {
+    const float* p = w + ((size_t)k * C + c) * 9;
+#pragma unroll
+    for (int i = 0; i < 9; ++i) g[i] = p[i];
+  } else {
+    const float* p = w + (size_t)c * 9 * K + k;
+#pragma unroll
+    for (int i = 0; i < 9; ++i) g[i] = p[(size_t)i * K];
+  }
+}
+
+// Reference layout Ww[c][p][k].  grid (ceil(K/256), C), block 256: thread = one (c,k).
+template <bool KCRS>
+__global__ void __launch_bounds__(256) fx_reference_layout(const float* __restrict__ w,
+                                                           float* __restrict__ Ww, int K,
+                                                           int C) {
+  const int k = blockIdx.x * 256 + threadIdx.x;
+  const int c = blockIdx.y;
+  if (k >= K) return;
+  float g[9], U[16];
+  load_filter<KCRS>(w, c, k, C, K, g);
+  fx_one(g, U);
+  float* o = Ww + (size_t)c * 16 * K + k;
+#pragma unroll
+  for (int p = 0; p < 16; ++p) o[(size_t)p * K] = U[p];
+}
+
+// MFMA-operand layout read by the fused kernel:
+//   Usw[kg][q][p][h][k32][s],  k = kg*32 + k32,  c = 4*q + 2*s + h
+// so that lane (h*32 + k32) of a wave fetches, with one 8-byte load per position p, the A
+// operand of two consecutive v_mfma_f32_32x32x2_f32 steps (channels 4q+h and 4q+2+h).
+// Thread = (k, q, h): transforms the two channels c = 4q+h and 4q+2+h and writes float2.
+// grid (ceil(K/128), C/4), block 256 = 2 h x 128 k.
+template <bool KCRS>
+__global__ void __launch_bounds__(256) fx_mfma_layout(const float* __restrict__ w,
+                                                      float* __restrict__ Usw, int K, int C) {
+  const int h = threadIdx.x >> 7;
+  const int k = blockIdx.x * 128 + (threadIdx.x & 127);
+  const int q = blockIdx.y;
+  if (k >= K) return;
+  float g0[9], g1[9], U0[16], U1[16];
+  load_filter<KCRS>(w, 4 * q + h, k, C, K, g0);
+  load_filter<KCRS>(w, 4 * q + 2 + h, k, C, K, g1);
+  fx_one(g0, U0);
+  fx_one(g1, U1);
+  const int kg = k >> 5, k32 = k & 31;
+  float2* o = reinterpret_cast<float2*>(Usw) +
+              (((size_t)kg * (C >> 2) + q) * 16) * 64 + h * 32 + k32;
+#pragma unroll
+  for (int p = 0; p < 16; ++p) o[(size_t)p * 64] = make_float2(U0[p], U1[p]);
+}
+
+}  // namespace opencnn

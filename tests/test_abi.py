@@ -1,0 +1,100 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol the header
+declares, validates arguments before touching a GPU, and the seeded generators behave."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "opencnn_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b([A-Za-z_][A-Za-z0-9_]*)\s*\(", text)) - {"defined"})
+
+
+def test_header_symbols_exported(ocn):
+    names = declared_functions()
+    assert "convolutionForward" in names and "opencnn_filter_transform" in names
+    handle = ctypes.CDLL(ocn.LIB_PATH)
+    for name in names:
+        assert hasattr(handle, name), f"{name} declared in include/opencnn_amd.h but not exported"
+    assert sorted(ocn.EXPORTED_SYMBOLS) == names  # the binding covers exactly the header
+
+
+def test_tiles_dim_and_workspace(ocn, oracle):
+    for w in (1, 2, 5, 7, 8, 14, 28, 56, 57, 224):
+        assert ocn.tiles_dim(w) == oracle.tiles_dim(w) == (w + 1) // 2
+    assert ocn.workspace_bytes(256, 256) == 256 * 256 * 16 * 4
+    assert ocn.workspace_bytes(0, 64) == 0
+
+
+def _call(ocn, **over):
+    """convolutionForward with dummy non-null pointers: validation must fail before launch."""
+    a = dict(N=32, C=8, H=8, W=8, K=64, R=3, S=3, m=2, alpha=4, tile=4)
+    a.update(over)
+    td = over.get("tiles_dim", ocn.tiles_dim(a["W"]))
+    oh, ow = over.get("out_h", a["H"]), over.get("out_w", a["W"])
+    on, oc = over.get("out_n", a["N"]), over.get("out_c", a["K"])
+    fc = over.get("filt_c", a["C"])
+    ptr = over.get("ptr", 0x1000)
+    return ocn.lib().convolutionForward(ptr, a["H"], a["W"], ptr, oh, ow, on, oc, ptr, ptr,
+                                        on * oc * oh * ow, td, a["N"], a["tile"], td * 4,
+                                        a["C"], a["K"], fc, a["R"], a["S"], a["alpha"], a["m"])
+
+
+@pytest.mark.parametrize("over", [
+    dict(N=48), dict(N=0), dict(K=48), dict(C=12), dict(C=0), dict(R=5), dict(S=1), dict(m=4),
+    dict(alpha=6), dict(tile=6), dict(H=8, W=10), dict(out_h=6), dict(out_n=64), dict(out_c=32),
+    dict(filt_c=16), dict(tiles_dim=3), dict(ptr=0), dict(N=1 << 20, H=56, W=56),
+])
+def test_unsupported_arguments_are_rejected(ocn, over):
+    # the reference mis-computes or returns garbage here (src/openCNN_winograd.cu:212-218);
+    # the drop-in must return hipErrorInvalidValue (1) and launch nothing
+    assert _call(ocn, **over) == 1
+    assert ocn.lib().opencnn_last_error() != b""
+
+
+def test_filter_transform_rejects_bad_arguments(ocn):
+    f = ocn.lib().opencnn_filter_transform
+    assert f(0x1000, 0x1000, 48, 8, 0, 0) == 1
+    assert f(0x1000, 0x1000, 64, 12, 0, 0) == 1
+    assert f(0x1000, 0x1000, 64, 8, 2, 0) == 1
+    assert f(0x1000, 0x1000, 64, 8, 0, 2) == 1
+    assert f(0, 0x1000, 64, 8, 0, 0) == 1
+
+
+def test_synth_layouts_agree(ocn):
+    N, C, H, W, K = 32, 8, 5, 6, 64
+    chwn = ocn.synth_input(N, C, H, W, seed=0x0C99)
+    nchw = ocn.synth_input(N, C, H, W, seed=0x0C99, layout=ocn.INPUT_NCHW)
+    assert np.array_equal(chwn, nchw.transpose(1, 2, 3, 0))
+    crsk = ocn.synth_filter(K, C, seed=0xF117)
+    kcrs = ocn.synth_filter(K, C, seed=0xF117, layout=ocn.FILTER_KCRS)
+    assert np.array_equal(crsk, kcrs.transpose(1, 2, 3, 0))
+
+
+def test_synth_distributions(ocn):
+    x = ocn.synth_input(64, 16, 14, 14, seed=1)
+    assert x.min() >= -1.0 and x.max() < 1.0 and abs(x.mean()) < 0.01
+    assert abs(x.var() - 1.0 / 3.0) < 0.01
+    relu = ocn.synth_input(64, 16, 14, 14, seed=1, p0=0.0, p1=1.0)
+    assert relu.min() >= 0.0 and relu.max() < 1.0
+    C = 64
+    g = ocn.synth_filter(128, C, seed=2)
+    assert abs(g.mean()) < 2e-3 and abs(g.std() / np.sqrt(2.0 / (9 * C)) - 1.0) < 0.02
+    assert not np.array_equal(x, ocn.synth_input(64, 16, 14, 14, seed=2))
+    assert np.array_equal(x, ocn.synth_input(64, 16, 14, 14, seed=1))
+
+
+def test_unswizzle_is_a_permutation(ocn):
+    C, K = 8, 64
+    a = np.arange(C * 16 * K, dtype=np.float32)
+    b = ocn.unswizzle_ww(a, C, K)
+    assert sorted(b.ravel().tolist()) == a.tolist()
+    # element (kg=1, q=1, p=3, h=1, k32=5, s=1) is c = 4+2+1 = 7, k = 37
+    idx = ((((1 * (C // 4) + 1) * 16 + 3) * 2 + 1) * 32 + 5) * 2 + 1
+    assert b[7, 3, 37] == a[idx]

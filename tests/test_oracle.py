@@ -1,0 +1,181 @@
+"""Pins the CPU oracle against what the mathematics fixes (the reference ships no tests,
+fixtures or golden vectors for this path): closed forms in fp64, textbook matrices,
+brute force on tiny inputs, exact-integer cases where every summation order agrees."""
+import numpy as np
+import pytest
+
+G = np.array([[1, 0, 0], [0.5, 0.5, 0.5], [0.5, -0.5, 0.5], [0, 0, 1]], dtype=np.float64)
+BT = np.array([[1, 0, -1, 0], [0, 1, 1, 0], [0, -1, 1, 0], [0, 1, 0, -1]], dtype=np.float64)
+AT = np.array([[1, 1, 1, 0], [0, 1, -1, -1]], dtype=np.float64)
+
+
+def brute_conv(x_chwn, w_crsk):
+    """Independent restatement: zero-pad, then einsum over shifted views (fp64)."""
+    x = np.asarray(x_chwn, dtype=np.float64)
+    w = np.asarray(w_crsk, dtype=np.float64)
+    C, H, W, N = x.shape
+    xp = np.zeros((C, H + 2, W + 2, N))
+    xp[:, 1:-1, 1:-1, :] = x
+    y = np.zeros((w.shape[3], H, W, N))
+    for r in range(3):
+        for s in range(3):
+            y += np.einsum("chwn,ck->khwn", xp[:, r:r + H, s:s + W, :], w[:, r, s, :])
+    return y
+
+
+def test_tiles_dim(oracle):
+    # ceil(ceil((W+2)/2)-1) for the sizes the reference sweeps (bench/bench.sh) and odd ones
+    for w, want in [(56, 28), (28, 14), (14, 7), (7, 4), (8, 4), (5, 3), (4, 2), (1, 1), (2, 1)]:
+        assert oracle.tiles_dim(w) == want
+
+
+def test_fx_closed_form(oracle):
+    rng = np.random.default_rng(1)
+    for _ in range(50):
+        g = rng.uniform(-1, 1, 9).astype(np.float32)
+        want = G @ g.reshape(3, 3).astype(np.float64) @ G.T
+        got = oracle.fx_one(g).reshape(4, 4)
+        np.testing.assert_allclose(got, want, rtol=0, atol=3e-7)
+
+
+def test_fx_delta_and_ones_exact(oracle):
+    # delta filter e_rs -> outer product of G's columns r and s; exact in fp32
+    for r in range(3):
+        for s in range(3):
+            g = np.zeros(9, np.float32)
+            g[r * 3 + s] = 1
+            want = np.outer(G[:, r], G[:, s]).astype(np.float32)
+            assert np.array_equal(oracle.fx_one(g).reshape(4, 4), want)
+    v = np.array([1, 1.5, 0.5, 1], np.float32)
+    assert np.array_equal(oracle.fx_one(np.ones(9, np.float32)).reshape(4, 4), np.outer(v, v))
+
+
+def test_fx_is_not_symmetric_under_transpose_mistake(oracle):
+    # a transposed operand (G^T g G) or swapped row/column pass would fail this
+    g = np.arange(9, dtype=np.float32)
+    want = (G @ g.reshape(3, 3).astype(np.float64) @ G.T).astype(np.float32)
+    got = oracle.fx_one(g).reshape(4, 4)
+    assert np.array_equal(got, want)  # small integers and halves: exact
+    assert not np.array_equal(got, got.T)
+
+
+def test_fx_tensor_layout(oracle):
+    rng = np.random.default_rng(2)
+    C, K = 8, 32
+    w = rng.integers(-4, 5, size=(C, 3, 3, K)).astype(np.float32)
+    got = oracle.fx(w)  # [C][16][K]
+    want = np.einsum("ir,crsk,js->cijk", G, w.astype(np.float64), G).reshape(C, 16, K)
+    assert np.array_equal(got, want.astype(np.float32))
+
+
+def test_input_transform_exact(oracle):
+    rng = np.random.default_rng(3)
+    for _ in range(50):
+        d = rng.integers(-8, 9, size=16).astype(np.float32)
+        want = BT @ d.reshape(4, 4).astype(np.float64) @ BT.T
+        assert np.array_equal(oracle.input_transform(d).reshape(4, 4), want.astype(np.float32))
+
+
+def test_output_transform_exact(oracle):
+    rng = np.random.default_rng(4)
+    for _ in range(50):
+        m = rng.integers(-8, 9, size=16).astype(np.float32)
+        want = AT @ m.reshape(4, 4).astype(np.float64) @ AT.T
+        assert np.array_equal(oracle.output_transform(m).reshape(2, 2), want.astype(np.float32))
+
+
+def test_winograd_identity_single_tile():
+    # the algebra the three transforms must satisfy together: A^T[(G g G^T).(B^T d B)]A = corr(d,g)
+    rng = np.random.default_rng(5)
+    d = rng.integers(-3, 4, size=(4, 4)).astype(np.float64)
+    g = rng.integers(-3, 4, size=(3, 3)).astype(np.float64)
+    y = AT @ ((G @ g @ G.T) * (BT @ d @ BT.T)) @ AT.T
+    want = np.array([[np.sum(d[a:a + 3, b:b + 3] * g) for b in range(2)] for a in range(2)])
+    np.testing.assert_allclose(y, want, atol=1e-12)
+
+
+@pytest.mark.parametrize("H,W", [(4, 4), (5, 5), (7, 7), (8, 8), (3, 6), (1, 1)])
+def test_direct_conv_vs_bruteforce(oracle, H, W):
+    rng = np.random.default_rng(10 + H * 16 + W)
+    N, C, K = 4, 5, 6
+    x = rng.uniform(-1, 1, (C, H, W, N)).astype(np.float32)
+    w = rng.uniform(-1, 1, (C, 3, 3, K)).astype(np.float32)
+    np.testing.assert_allclose(oracle.direct_conv_f64(x, w), brute_conv(x, w), rtol=0, atol=1e-12)
+
+
+def test_direct_conv_impulse(oracle):
+    # single input pixel: the output neighbourhood carries the filter taps, index-reversed
+    # (cross-correlation: y[h0-(r-1), w0-(s-1)] = g[r][s]); pins every stride of all layouts
+    N, C, K, H, W = 3, 4, 5, 6, 7
+    rng = np.random.default_rng(6)
+    w = rng.uniform(-1, 1, (C, 3, 3, K)).astype(np.float32)
+    for (c0, h0, w0, n0) in [(0, 0, 0, 0), (3, 5, 6, 2), (1, 2, 3, 1)]:
+        x = np.zeros((C, H, W, N), np.float32)
+        x[c0, h0, w0, n0] = 1.0
+        y = oracle.direct_conv_f64(x, w)
+        want = np.zeros_like(y)
+        for r in range(3):
+            for s in range(3):
+                hh, ww = h0 - (r - 1), w0 - (s - 1)
+                if 0 <= hh < H and 0 <= ww < W:
+                    want[:, hh, ww, n0] = w[c0, r, s, :]
+        assert np.array_equal(y, want)
+
+
+@pytest.mark.parametrize("H", [4, 5, 7, 8, 14])
+def test_winograd_restatement_vs_direct(oracle, H):
+    # odd and even sizes: a wrong mask or tile origin gives O(1) border errors
+    rng = np.random.default_rng(20 + H)
+    N, C, K = 4, 8, 16
+    x = rng.uniform(-1, 1, (C, H, H, N)).astype(np.float32)
+    w = rng.normal(0, np.sqrt(2.0 / (9 * C)), (C, 3, 3, K)).astype(np.float32)
+    y = oracle.winograd_f32(x, w)
+    assert not np.isnan(y).any()  # every output element written
+    rel, max_abs, max_ref = oracle.compare(y, oracle.direct_conv_f64(x, w))
+    assert rel <= 5e-7 and max_abs <= 1e-6 * max(max_ref, 1.0)
+
+
+def test_winograd_restatement_exact_on_integers(oracle):
+    # x in {-2..2}, g in {-2,0,2}: U is a multiple of 1/2, every partial sum is exactly
+    # representable, so the Winograd result equals the direct result bit for bit.
+    rng = np.random.default_rng(7)
+    N, C, K, H = 4, 8, 8, 7
+    x = rng.integers(-2, 3, (C, H, H, N)).astype(np.float32)
+    w = (2 * rng.integers(-1, 2, (C, 3, 3, K))).astype(np.float32)
+    y = oracle.winograd_f32(x, w)
+    assert np.array_equal(y.astype(np.float64), oracle.direct_conv_f64(x, w))
+
+
+def test_winograd_linearity(oracle):
+    rng = np.random.default_rng(8)
+    N, C, K, H = 2, 8, 8, 6
+    x1 = rng.integers(-2, 3, (C, H, H, N)).astype(np.float32)
+    x2 = rng.integers(-2, 3, (C, H, H, N)).astype(np.float32)
+    w = (2 * rng.integers(-1, 2, (C, 3, 3, K))).astype(np.float32)
+    lhs = oracle.winograd_f32(2 * x1 - 3 * x2, w)
+    rhs = 2 * oracle.winograd_f32(x1, w) - 3 * oracle.winograd_f32(x2, w)
+    assert np.array_equal(lhs, rhs)
+
+
+def test_rounding_helpers(oracle):
+    # fp16 / bf16 round-to-nearest-even against numpy's float16 and a manual bf16
+    rng = np.random.default_rng(9)
+    vals = np.concatenate([rng.uniform(-4, 4, 200), rng.uniform(-1e-6, 1e-6, 50),
+                           [0.0, 1.0, 65504.0, 70000.0, 2.0 ** -24, 2.0 ** -25, 1.0009765625]])
+    for v in vals.astype(np.float32):
+        with np.errstate(over="ignore"):
+            assert oracle.round_operand(v, 1) == float(np.float32(np.float16(v)))
+        u = np.float32(v).view(np.uint32)
+        bf = np.uint32((int(u) + 0x7FFF + ((int(u) >> 16) & 1)) & 0xFFFF0000).view(np.float32)
+        assert oracle.round_operand(v, 2) == float(bf)
+
+
+@pytest.mark.parametrize("quant,bound", [(1, 2e-3), (2, 1.5e-2)])
+def test_quantised_restatement_vs_direct(oracle, quant, bound):
+    # fp16 / bf16 GEMM operands: unit round-offs 2^-11 / 2^-8 on both operands
+    rng = np.random.default_rng(30 + quant)
+    N, C, K, H = 4, 16, 16, 7
+    x = rng.uniform(-1, 1, (C, H, H, N)).astype(np.float32)
+    w = rng.normal(0, np.sqrt(2.0 / (9 * C)), (C, 3, 3, K)).astype(np.float32)
+    rel, _, _ = oracle.compare(oracle.winograd_f32(x, w, quant), oracle.direct_conv_f64(x, w))
+    assert 1e-6 < rel <= bound  # quantisation visible, inside the stated bound

@@ -1,0 +1,231 @@
+"""GPU parity tests: the HIP path, called through the C ABI, against the CPU oracle.
+
+Tolerances (fp32 path): relative L2 <= 1e-5 and max-abs <= 1e-4 * max|y| against the
+reference-order fp32 Winograd restatement; relative L2 <= 1e-3 against the fp64 direct
+convolution.  Filter transform and exact-integer cases: bit-exact.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+REL_L2_WINOGRAD = 1e-5
+MAX_ABS_WINOGRAD = 1e-4  # times max|y|
+REL_L2_DIRECT = 1e-3
+
+SEED_X, SEED_W = 0x0C99, 0xF117
+
+# (name, N, C, H, K, input range, filter distribution) — the benchmark configurations
+CONFIGS = [
+    ("plumbing", 32, 8, 8, 64, (-1.0, 1.0), "uniform"),
+    ("resnet_56", 64, 64, 56, 64, (-1.0, 1.0), "he"),
+    ("resnet_28", 128, 128, 28, 128, (-1.0, 1.0), "he"),
+    ("deep_14", 128, 256, 14, 256, (0.0, 1.0), "he"),
+    ("deep_7", 128, 512, 7, 512, (0.0, 1.0), "he"),
+]
+
+
+def make_tensors(ocn, N, C, H, W, K, xr=(-1.0, 1.0), filt="he"):
+    x = ocn.synth_input(N, C, H, W, seed=SEED_X, p0=xr[0], p1=xr[1])
+    if filt == "he":
+        w = ocn.synth_filter(K, C, seed=SEED_W)
+    else:
+        w = ocn.synth_filter(K, C, seed=SEED_W, dist=ocn.DIST_UNIFORM, p0=-1.0, p1=1.0)
+    return x, w
+
+
+class Runner:
+    """Owns device buffers (with guard bands around the output) and calls the C ABI."""
+
+    GUARD = 4096
+
+    def __init__(self, ocn, torch, x, w):
+        self.ocn, self.torch = ocn, torch
+        self.C, self.H, self.W, self.N = x.shape
+        self.K = w.shape[3]
+        dev = torch.device("cuda:0")
+        self.xd = torch.from_numpy(np.ascontiguousarray(x)).to(dev)
+        self.wd = torch.from_numpy(np.ascontiguousarray(w)).to(dev)
+        self.ws = torch.empty(ocn.workspace_bytes(self.C, self.K) // 4, device=dev)
+        self.n_out = self.K * self.H * self.W * self.N
+        self.raw = torch.full((self.n_out + 2 * self.GUARD,), float("nan"), device=dev)
+        self.yd = self.raw[self.GUARD:self.GUARD + self.n_out]
+
+    def dropin(self):
+        """The reference's call, argument for argument (src/openCNN_winograd.cu:429-431)."""
+        o, td = self.ocn, self.ocn.tiles_dim(self.W)
+        o.convolutionForward(self.xd, self.H, self.W, self.wd, self.H, self.W, self.N, self.K,
+                             self.yd, self.ws, self.n_out, td, self.N, 4, td * 4, self.C,
+                             self.K, self.C, 3, 3, 4, 2)
+        return self.result()
+
+    def split(self):
+        """Filter transform once, then the fused kernel (allows H != W)."""
+        o = self.ocn
+        o.filter_transform(self.wd, self.ws, self.K, self.C, o.FILTER_CRSK, o.WW_MFMA)
+        o.conv_forward_pretransformed(self.xd, self.ws, self.yd, self.N, self.C, self.H,
+                                      self.W, self.K)
+        return self.result()
+
+    def result(self):
+        self.torch.cuda.synchronize()
+        raw = self.raw.cpu().numpy()
+        g = self.GUARD
+        assert np.isnan(raw[:g]).all() and np.isnan(raw[-g:]).all(), "wrote outside the output"
+        return raw[g:-g].reshape(self.K, self.H, self.W, self.N).copy()
+
+
+def check_against_oracle(oracle, y, x, w):
+    assert not np.isnan(y).any(), "an output element was never written"
+    rel, max_abs, max_ref = oracle.compare(y, oracle.winograd_f32(x, w))
+    assert rel <= REL_L2_WINOGRAD, f"rel-L2 vs fp32 Winograd restatement {rel:.3e}"
+    assert max_abs <= MAX_ABS_WINOGRAD * max_ref, f"max-abs {max_abs:.3e} vs max|y| {max_ref:.3e}"
+    rel64, _, _ = oracle.compare(y, oracle.direct_conv_f64(x, w))
+    assert rel64 <= REL_L2_DIRECT, f"rel-L2 vs fp64 direct convolution {rel64:.3e}"
+    return rel, rel64
+
+
+# ---------------------------------------------------------------- filter transform (FX)
+
+@pytest.mark.parametrize("C,K", [(8, 64), (64, 64), (128, 128), (256, 256), (512, 512), (8, 32), (24, 96)])
+def test_fx_bit_exact(ocn, oracle, torch_gpu, C, K):
+    torch = torch_gpu
+    print(f"fx C={C} K={K}", flush=True)
+    crsk = ocn.synth_filter(K, C, seed=SEED_W)
+    kcrs = ocn.synth_filter(K, C, seed=SEED_W, layout=ocn.FILTER_KCRS)
+    want = oracle.fx(crsk)
+    for host, layout in ((crsk, ocn.FILTER_CRSK), (kcrs, ocn.FILTER_KCRS)):
+        wd = torch.from_numpy(host).cuda()
+        out = torch.full((C * 16 * K,), float("nan"), device="cuda")
+        ocn.filter_transform(wd, out, K, C, layout, ocn.WW_REFERENCE)
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy().reshape(C, 16, K), want)
+        out.fill_(float("nan"))
+        ocn.filter_transform(wd, out, K, C, layout, ocn.WW_MFMA)
+        torch.cuda.synchronize()
+        assert np.array_equal(ocn.unswizzle_ww(out.cpu().numpy(), C, K), want)
+
+
+# ---------------------------------------------------------------- whole path, benchmark sizes
+
+@pytest.mark.parametrize("name,N,C,H,K,xr,filt", CONFIGS, ids=[c[0] for c in CONFIGS])
+def test_benchmark_configs(ocn, oracle, torch_gpu, name, N, C, H, K, xr, filt):
+    print(f"config {name} N={N} C={C} H={H} K={K}", flush=True)
+    x, w = make_tensors(ocn, N, C, H, H, K, xr, filt)
+    y = Runner(ocn, torch_gpu, x, w).dropin()
+    rel, rel64 = check_against_oracle(oracle, y, x, w)
+    print(f"  rel-L2 vs Winograd restatement {rel:.2e}, vs fp64 direct {rel64:.2e}", flush=True)
+
+
+@pytest.mark.parametrize("N", [32, 64, 96, 128])
+def test_reference_sweep_batch_sizes(ocn, oracle, torch_gpu, N):
+    # the batch sizes of the reference's sweep (bench/bench.sh:3-21) on its 14x14 layer, C=K cut to 64
+    print(f"sweep N={N}", flush=True)
+    x, w = make_tensors(ocn, N, 64, 14, 14, 64)
+    check_against_oracle(oracle, Runner(ocn, torch_gpu, x, w).dropin(), x, w)
+
+
+# ---------------------------------------------------------------- edges
+
+@pytest.mark.parametrize("H", [1, 2, 3, 4, 5, 6, 7, 9, 13])
+def test_small_square_sizes(ocn, oracle, torch_gpu, H):
+    # odd sizes exercise both mask sets of the reference
+    # (src/convolutionForward_32x64x8.cu:179-183, src/store_and_transform_output_optSTS64.cuh:65-67)
+    print(f"square H={H}", flush=True)
+    x, w = make_tensors(ocn, 32, 8, H, H, 32)
+    check_against_oracle(oracle, Runner(ocn, torch_gpu, x, w).dropin(), x, w)
+
+
+@pytest.mark.parametrize("H,W", [(3, 8), (8, 3), (5, 12), (14, 7), (1, 9)])
+def test_rectangular_sizes(ocn, oracle, torch_gpu, H, W):
+    # beyond the reference (it only models H == W): checked against the fp64 direct convolution
+    print(f"rect H={H} W={W}", flush=True)
+    x, w = make_tensors(ocn, 32, 16, H, W, 64)
+    y = Runner(ocn, torch_gpu, x, w).split()
+    assert not np.isnan(y).any()
+    rel64, _, _ = oracle.compare(y, oracle.direct_conv_f64(x, w))
+    assert rel64 <= 1e-5
+
+
+def test_ragged_column_blocks(ocn, oracle, torch_gpu):
+    # 25 tiles x 1 batch group = 25 wave tiles: the last workgroup has idle waves
+    print("ragged", flush=True)
+    x, w = make_tensors(ocn, 32, 8, 10, 10, 96)
+    check_against_oracle(oracle, Runner(ocn, torch_gpu, x, w).dropin(), x, w)
+
+
+# ---------------------------------------------------------------- exact and structural properties
+
+def test_integer_tensors_bit_exact(ocn, oracle, torch_gpu):
+    # x in {-2..2}, g in {-2,0,2}: every summation order gives the same fp32 result, so the
+    # MFMA path must equal the fp64 direct convolution bit for bit (odd size: masks included)
+    print("integers", flush=True)
+    rng = np.random.default_rng(7)
+    N, C, K, H = 64, 64, 64, 7
+    x = rng.integers(-2, 3, (C, H, H, N)).astype(np.float32)
+    w = (2 * rng.integers(-1, 2, (C, 3, 3, K))).astype(np.float32)
+    y = Runner(ocn, torch_gpu, x, w).dropin()
+    assert np.array_equal(y.astype(np.float64), oracle.direct_conv_f64(x, w))
+    assert np.array_equal(y, oracle.winograd_f32(x, w))
+
+
+def test_impulse_reproduces_filter_taps(ocn, torch_gpu):
+    # one non-zero input pixel: y[:, h0-(r-1), w0-(s-1), n0] = g[c0][r][s][:]; pins all strides
+    print("impulse", flush=True)
+    N, C, K, H = 32, 8, 32, 6
+    w = ocn.synth_filter(K, C, seed=SEED_W)
+    for (c0, h0, w0, n0) in [(0, 0, 0, 0), (7, 5, 5, 31), (3, 2, 4, 17)]:
+        x = np.zeros((C, H, H, N), np.float32)
+        x[c0, h0, w0, n0] = 1.0
+        y = Runner(ocn, torch_gpu, x, w).dropin()
+        want = np.zeros_like(y)
+        for r in range(3):
+            for s in range(3):
+                hh, ww = h0 - (r - 1), w0 - (s - 1)
+                if 0 <= hh < H and 0 <= ww < H:
+                    want[:, hh, ww, n0] = w[c0, r, s, :]
+        np.testing.assert_allclose(y, want, rtol=0, atol=2e-7)
+
+
+def test_linearity_at_full_size(ocn, torch_gpu):
+    # size-independent property on the 28x28 benchmark layer: conv(2a-3b) = 2conv(a)-3conv(b)
+    print("linearity", flush=True)
+    N, C, H, K = 128, 128, 28, 128
+    a = ocn.synth_input(N, C, H, H, seed=11)
+    b = ocn.synth_input(N, C, H, H, seed=12)
+    w = ocn.synth_filter(K, C, seed=SEED_W)
+    ya = Runner(ocn, torch_gpu, a, w).dropin()
+    yb = Runner(ocn, torch_gpu, b, w).dropin()
+    yc = Runner(ocn, torch_gpu, 2 * a - 3 * b, w).dropin()
+    want = 2 * ya.astype(np.float64) - 3 * yb.astype(np.float64)
+    err = np.linalg.norm((yc - want).ravel()) / np.linalg.norm(want.ravel())
+    assert err <= 1e-6, err
+
+
+def test_repeated_calls_are_identical_and_split_matches_dropin(ocn, torch_gpu):
+    print("repeat", flush=True)
+    x, w = make_tensors(ocn, 64, 64, 14, 14, 128)
+    r = Runner(ocn, torch_gpu, x, w)
+    y1 = r.dropin()
+    y2 = r.dropin()  # same Ww scratch, back to back (stream ordered)
+    assert np.array_equal(y1, y2)
+    assert np.array_equal(y1, r.split())
+
+
+def test_non_default_stream(ocn, oracle, torch_gpu):
+    print("stream", flush=True)
+    torch = torch_gpu
+    x, w = make_tensors(ocn, 32, 16, 9, 9, 64)
+    r = Runner(ocn, torch, x, w)
+    s = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    try:
+        ocn.set_stream(s)
+        y = r.dropin()
+    finally:
+        ocn.set_stream(None)
+    check_against_oracle(oracle, y, x, w)
+
+
+def test_init_accepts_this_device(ocn, torch_gpu):
+    ocn.init()
