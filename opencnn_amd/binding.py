@@ -86,6 +86,14 @@ def load_library(path: str = LIB_PATH) -> ctypes.CDLL:
         raise ImportError(
             f"{path} is missing: build it with `make -C opencnn_amd/csrc` "
             "(or __graft_entry__.build()); opencnn_amd has no non-HIP path")
+    # One HIP runtime per process: torch ships its own libamdhip64 (same SONAME as ROCm's).
+    # Importing torch first makes the dynamic loader resolve this library's dependency to the
+    # copy torch already mapped; loaded in the other order the process ends up with two
+    # runtimes and the second one reports hipErrorNoDevice.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     handle = ctypes.CDLL(path)
     for name, (restype, argtypes) in EXPORTED_SYMBOLS.items():
         fn = getattr(handle, name)  # AttributeError if the symbol is not exported
