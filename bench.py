@@ -1,0 +1,206 @@
+#!/usr/bin/env python3
+"""Benchmark of the Winograd F(2x2,3x3) forward convolution on one MI355X.
+
+A "step" is one call of the reference's entry point ``convolutionForward`` (filter
+transform + fused kernel, the quantity the reference times at
+src/openCNN_winograd.cu:426-444) on one seeded synthetic layer resident in HBM.
+
+Prints ONE JSON line: effective TFLOP/s (direct-convolution FLOPs 2*N*K*C*H*W*9 per
+step), ms per layer, the roofline of the dominant kernel (fp32 MFMA, algorithmic
+flops 32*N*T*C*K per launch) and a CPU baseline (the fp64 direct convolution of the
+oracle on the host cores).  ``layers`` repeats the figures for every fp32 layer of the
+benchmark set; only ``config.workload`` is the timed K-step region.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
+PEAK_HBM_GBS = 8000.0
+
+# name -> (N, C, H=W, K, input range, filter distribution)
+LAYERS = {
+    "plumbing_n32_c8_h8_k64": (32, 8, 8, 64, (-1.0, 1.0), "uniform"),
+    "resnet_n64_c64_h56_k64": (64, 64, 56, 64, (-1.0, 1.0), "he"),
+    "resnet_n128_c128_h28_k128": (128, 128, 28, 128, (-1.0, 1.0), "he"),
+    "deep_n128_c256_h14_k256": (128, 256, 14, 256, (0.0, 1.0), "he"),
+    "deep_n128_c512_h7_k512": (128, 512, 7, 512, (0.0, 1.0), "he"),
+}
+DEFAULT_WORKLOAD = "resnet_n64_c64_h56_k64"
+
+# HBM bytes per launch of the fused kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# (profiles/), or None where not measured yet.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def work(N, C, H, K):
+    T = ((H + 1) // 2) ** 2
+    flops_direct = 2.0 * N * K * C * H * H * 9
+    flops_mfma = 32.0 * N * T * C * K
+    bytes_min = 4.0 * (N * C * H * H + 9 * K * C + 2 * 16 * K * C + N * K * H * H)
+    return flops_direct, flops_mfma, bytes_min
+
+
+class Layer:
+    def __init__(self, ocn, torch, name):
+        self.name = name
+        self.N, self.C, self.H, self.K, xr, filt = LAYERS[name]
+        self.x_host = ocn.synth_input(self.N, self.C, self.H, self.H, seed=0x0C99, p0=xr[0], p1=xr[1])
+        if filt == "he":
+            self.w_host = ocn.synth_filter(self.K, self.C, seed=0xF117)
+        else:
+            self.w_host = ocn.synth_filter(self.K, self.C, seed=0xF117, dist=ocn.DIST_UNIFORM,
+                                           p0=-1.0, p1=1.0)
+        dev = torch.device("cuda:0")
+        self.x = torch.from_numpy(self.x_host).to(dev)
+        self.w = torch.from_numpy(self.w_host).to(dev)
+        self.y = torch.empty((self.K, self.H, self.H, self.N), device=dev)
+        self.ws = torch.empty(ocn.workspace_bytes(self.C, self.K) // 4, device=dev)
+        self.ocn = ocn
+        self.td = ocn.tiles_dim(self.H)
+
+    def step(self):
+        o = self
+        self.ocn.convolutionForward(o.x, o.H, o.H, o.w, o.H, o.H, o.N, o.K, o.y, o.ws,
+                                    o.K * o.N * o.H * o.H, o.td, o.N, 4, o.td * 4, o.C, o.K,
+                                    o.C, 3, 3, 4, 2)
+
+    def kernel_times(self, warmup, iters):
+        """HIP-event mean ms per call on the library's stream: (fx+main, main, fx)."""
+        return self.ocn.time_forward(self.x, self.w, self.y, self.ws, self.N, self.C, self.H,
+                                     self.H, self.K, warmup=warmup, iters=iters)
+
+
+def cpu_baseline(layer):
+    """The oracle's fp64 direct convolution on the host cores, one warm + one timed pass."""
+    from oracle import oracle
+
+    # bounded sample: the layer itself when it is small enough, else its first images
+    n = layer.N
+    x = layer.x_host[..., :n]
+    oracle.direct_conv_f64(x[..., :32], layer.w_host)  # warm (threads, pages)
+    t0 = time.perf_counter()
+    y = oracle.direct_conv_f64(x, layer.w_host)
+    dt = time.perf_counter() - t0
+    flops = 2.0 * n * layer.K * layer.C * layer.H * layer.H * 9
+    return y, {
+        "value": flops / dt / 1e12,
+        "unit": "TFLOP/s",
+        "cores": oracle.num_threads(),
+        "kind": "port",
+        "sample": f"fp64 direct convolution of the whole {layer.name} layer ({n} images), "
+                  f"1 warm-up + 1 timed pass, {dt * 1e3:.0f} ms",
+        "ms_per_layer": dt * 1e3,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(LAYERS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-layers", action="store_true", help="skip the per-layer table")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (a single layer on one device, no "
+                 "collectives); run it with --gpus 1")
+
+    import torch
+
+    import opencnn_amd as ocn
+
+    ocn.load_library()  # raises if the HIP library is not built: there is no other path
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    ocn.init()
+
+    layer = Layer(ocn, torch, args.workload)
+    fd, fm, bmin = work(layer.N, layer.C, layer.H, layer.K)
+
+    for _ in range(args.warmup):
+        layer.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        layer.step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_step = dt * 1e3 / args.steps
+
+    # dominant kernel, HIP events on the launch stream, same number of launches
+    _, ms_main, ms_fx = layer.kernel_times(args.warmup, args.steps)
+    achieved = fm / (ms_main * 1e-3) / 1e12
+    traffic = MEASURED_TRAFFIC_BYTES.get(layer.name)
+
+    out = {
+        "metric": "effective TFLOP/s (direct-conv FLOPs 2*N*K*C*H*W*9) of one 3x3 fp32 layer, "
+                  "filter transform + fused Winograd kernel per call",
+        "value": fd / (ms_step * 1e-3) / 1e12,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": layer.name, "N": layer.N, "C": layer.C, "H": layer.H,
+                   "W": layer.H, "K": layer.K, "pad": 1, "stride": 1,
+                   "layout": "CHWN in, CRSK filters, KHWN out"},
+        "roofline": {
+            "kernel": "wino_f32_fused",
+            "bound": "mfma",
+            "achieved": achieved,
+            "peak": PEAK_FP32_MFMA_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
+            "traffic": traffic,
+            "flops_per_launch": fm,
+            "ms_per_launch": ms_main,
+            "hbm_min_bytes": bmin,
+            "hbm_gbs_at_min_bytes": bmin / (ms_step * 1e-3) / 1e9,
+            "fx_ms_per_launch": ms_fx,
+        },
+    }
+
+    if not args.no_cpu:
+        from oracle import oracle
+
+        y_ref, base = cpu_baseline(layer)
+        out["cpu_baseline"] = base
+        rel, max_abs, max_ref = oracle.compare(layer.y.cpu().numpy(), y_ref)
+        out["check"] = {"rel_l2_vs_fp64_direct": rel, "max_abs": max_abs, "max_ref": max_ref}
+        if not rel <= 1e-3:
+            sys.exit(f"bench.py: GPU result differs from the fp64 direct convolution (rel-L2 {rel})")
+
+    if not args.no_layers:
+        rows = []
+        for name in LAYERS:
+            lay = layer if name == layer.name else Layer(ocn, torch, name)
+            tot, mn, fx = lay.kernel_times(3, 50)
+            d, m, b = work(lay.N, lay.C, lay.H, lay.K)
+            rows.append({
+                "workload": name, "ms_per_layer": tot, "ms_fused_kernel": mn, "ms_filter_transform": fx,
+                "effective_tflops": d / (tot * 1e-3) / 1e12,
+                "mfma_tflops": m / (mn * 1e-3) / 1e12,
+                "mfma_frac_of_peak": m / (mn * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS,
+                "hbm_gbs_at_min_bytes": b / (tot * 1e-3) / 1e9,
+            })
+            del lay
+        out["layers"] = rows
+
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -94,7 +94,7 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   a.nblocks = (int)nblocks;
   const int per_xcd = (a.nblocks + 7) / 8;
   dim3 grid(per_xcd * 8), block(256);
-  opencnn::wino_f32_fused<2><<<grid, block, 0, st>>>(a);
+  opencnn::wino_f32_fused<<<grid, block, 0, st>>>(a);
   return (int)hipGetLastError();
 }
 

@@ -88,10 +88,14 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, unsig
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, kBufferFlags);
 }
 
-// NBUF = number of 4x4 patches a lane keeps in flight ahead of the MFMA step that uses them.
-template <int NBUF>
+// One MFMA step = two input channels.  Software pipeline, per step t (all in registers):
+//   top     issue the 16 patch loads of step t+2 (and, every other step, the 16 filter
+//           loads of the quad after next);
+//   body    16 MFMAs of step t, interleaved with the 32 add/sub that turn the patch of
+//           step t+1 (loaded one step ago) into the next B operands.
+// The scheduling barriers keep hipcc from sinking the loads down to their first use (it
+// does so to save registers, which exposes the full memory latency once per step).
 __global__ void __launch_bounds__(256) wino_f32_fused(ConvArgs a) {
-  static_assert(NBUF == 1 || NBUF == 2 || NBUF == 4, "NBUF must divide 4");
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 
@@ -153,33 +157,40 @@ __global__ void __launch_bounds__(256) wino_f32_fused(ConvArgs a) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[p][r] = 0.0f;
 
-  v2f u[2][16];
-  float d[NBUF][16];
-  float v[2][16];
+  v2f u[2][16];    // filter operands of the current / next quad
+  float d[2][16];  // patches in flight: d[t&1] holds the patch of step t
+  float v[2][16];  // B operands: v[t&1] holds the transformed patch of step t
 
-  // prologue
+  // prologue: patch 0 -> v[0]; patch 1 in flight in d[1]; quad 0 in u[0]
   load_u(u[0], 0);
-  {
-    float d0[16];
-    load_patch(d0, 0);
-#pragma unroll
-    for (int m = 1; m <= NBUF; ++m) load_patch(d[m % NBUF], m);
-    input_transform(d0, v[0]);
-  }
+  load_patch(d[0], 0);
+  load_patch(d[1], 1);
+  input_transform(d[0], v[0]);
 
   const int octs = a.C >> 3;
   for (int oct = 0; oct < octs; ++oct) {
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       const int t = oct * 4 + s;
+      // d[t&1] was consumed by the transform of the previous step: refill it with step t+2
+      load_patch(d[s & 1], t + 2);
       if (s == 0) load_u(u[1], 2 * oct + 1);
       if (s == 2) load_u(u[0], 2 * oct + 2);
-      // transform the next step's patch while this step's MFMAs run
-      input_transform(d[(s + 1) % NBUF], v[(s + 1) & 1]);
-      load_patch(d[(s + 1) % NBUF], t + 1 + NBUF);
+      __builtin_amdgcn_sched_barrier(0);
+      input_transform(d[(s + 1) & 1], v[(s + 1) & 1]);
+      // Anchor: the next B operands must exist when this region ends, or LLVM sinks the
+      // transform into the next step, in front of the MFMAs that need it.
+#pragma unroll
+      for (int p = 0; p < 16; ++p) asm volatile("" : "+v"(v[(s + 1) & 1][p]));
 #pragma unroll
       for (int p = 0; p < 16; ++p)
         acc[p] = __builtin_amdgcn_mfma_f32_32x32x2f32(u[s >> 1][p][s & 1], v[s & 1][p], acc[p], 0, 0, 0);
+#pragma unroll
+      for (int p = 0; p < 16; ++p) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);  // two VALU of the next transform
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 
