@@ -31,7 +31,7 @@ extern "C" {
 /* Layout of the transformed-filter buffer written by opencnn_filter_transform. */
 enum {
   OPENCNN_WW_REFERENCE = 0, /* [filt_c][16][filt_k], position p = i*4+j (src/FX_m2.cu:84) */
-  OPENCNN_WW_MFMA = 1       /* [filt_k/32][filt_c/4][16][2][32][2]: what the fused kernel reads */
+  OPENCNN_WW_MFMA = 1       /* [filt_k/32][filt_c/4][16][2][32][2]: what the fused kernels read */
 };
 
 /* Layout of the 3x3 filters handed to the library. */
@@ -97,6 +97,19 @@ size_t opencnn_workspace_bytes(int filt_c, int filt_k);
  * NULL selects the null stream, which is what the reference launches on
  * (src/convolutionForward_32x64x8.cu:274,281). */
 int opencnn_set_stream(void *stream);
+
+/*
+ * Which fused kernel later calls launch.  The reference picks its variant at compile time
+ * (-DBASE / -DOPTSTS64 / -DOPTSTS64_CMP / -DOPTLDS64, Makefile:3,8); here it is a run-time
+ * switch so both can be measured in one process.
+ *   OPENCNN_KERNEL_AUTO      the LDS variant when filt_k % 64 == 0, else the register variant
+ *   OPENCNN_KERNEL_REGISTER  every wave transforms its own input patches; no LDS, no barriers
+ *   OPENCNN_KERNEL_LDS       the waves of a workgroup that share a column tile split the input
+ *                            transform and exchange it through LDS (needs filt_k % 64 == 0,
+ *                            otherwise later launches return hipErrorInvalidValue)
+ */
+enum { OPENCNN_KERNEL_AUTO = 0, OPENCNN_KERNEL_REGISTER = 1, OPENCNN_KERNEL_LDS = 2 };
+int opencnn_set_kernel_variant(int variant);
 
 /*
  * The reference's FX kernel as a call of its own (src/FX_m2.cu:51-91, launched at

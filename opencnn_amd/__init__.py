@@ -17,6 +17,10 @@ from .binding import (  # noqa: F401
     lib,
     load_library,
     set_stream,
+    set_kernel_variant,
+    KERNEL_AUTO,
+    KERNEL_REGISTER,
+    KERNEL_LDS,
     synth_filter,
     synth_input,
     tiles_dim,

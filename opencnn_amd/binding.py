@@ -20,6 +20,7 @@ WW_REFERENCE, WW_MFMA = 0, 1
 FILTER_CRSK, FILTER_KCRS = 0, 1
 INPUT_CHWN, INPUT_NCHW = 0, 1
 DIST_UNIFORM, DIST_NORMAL = 0, 1
+KERNEL_AUTO, KERNEL_REGISTER, KERNEL_LDS = 0, 1, 2
 
 _c_int, _c_float_p, _c_void_p = ctypes.c_int, ctypes.POINTER(ctypes.c_float), ctypes.c_void_p
 
@@ -41,6 +42,7 @@ EXPORTED_SYMBOLS = {
     "opencnn_tiles_dim": (_c_int, [_c_int]),
     "opencnn_workspace_bytes": (ctypes.c_size_t, [_c_int, _c_int]),
     "opencnn_set_stream": (_c_int, [_c_void_p]),
+    "opencnn_set_kernel_variant": (_c_int, [_c_int]),
     "opencnn_filter_transform": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int]),
     "opencnn_conv_forward_pretransformed": (
         _c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int]),
@@ -155,6 +157,11 @@ def set_stream(stream) -> None:
     """Select the stream of later calls: a torch.cuda.Stream, a raw handle or None."""
     handle = 0 if stream is None else getattr(stream, "cuda_stream", stream)
     _check("opencnn_set_stream", lib().opencnn_set_stream(handle))
+
+
+def set_kernel_variant(variant: int) -> None:
+    """KERNEL_AUTO, KERNEL_REGISTER or KERNEL_LDS for later launches."""
+    _check("opencnn_set_kernel_variant", lib().opencnn_set_kernel_variant(variant))
 
 
 def convolutionForward(k, in_h, in_w, w, out_h, out_w, out_n, out_c, C, Ww, n, tiles_dim,

@@ -15,6 +15,7 @@
 namespace {
 
 std::atomic<hipStream_t> g_stream{nullptr};
+std::atomic<int> g_variant{OPENCNN_KERNEL_AUTO};
 thread_local const char* t_last_error = "";
 
 int fail(const char* what) {
@@ -88,13 +89,30 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   a.ngroups = in_n / 32;
   a.colgroups = a.tiles_h * a.tiles_w * a.ngroups;
   a.kgroups = filt_k / 32;
-  const long long colblocks = (a.colgroups + 3) / 4;
-  const long long nblocks = colblocks * a.kgroups;
+  // Waves per workgroup that share one column tile (and split its input transform).
+  int kw = 1;
+  const int variant = g_variant.load();
+  if (variant != OPENCNN_KERNEL_REGISTER) kw = filt_k % 128 == 0 ? 4 : (filt_k % 64 == 0 ? 2 : 1);
+  if (variant == OPENCNN_KERNEL_LDS) REQUIRE(kw > 1);
+  const int cw = 4 / kw;
+  const long long colblocks = (a.colgroups + cw - 1) / cw;
+  const long long nblocks = colblocks * (a.kgroups / kw);
   REQUIRE(nblocks <= kMaxElems / 8);
   a.nblocks = (int)nblocks;
   const int per_xcd = (a.nblocks + 7) / 8;
   dim3 grid(per_xcd * 8), block(256);
-  opencnn::wino_f32_fused<<<grid, block, 0, st>>>(a);
+  const size_t lds_bytes = (size_t)cw * 2 * 4 * 16 * 64 * sizeof(float);
+  if (kw == 4)
+    opencnn::wino_f32_fused_lds<4><<<grid, block, lds_bytes, st>>>(a);
+  else if (kw == 2) {
+    // 96 KB of LDS: above the 64 KB a kernel gets without asking (gfx950 has 160 KB per CU)
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&opencnn::wino_f32_fused_lds<2>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) return (int)e;
+    opencnn::wino_f32_fused_lds<2><<<grid, block, lds_bytes, st>>>(a);
+  }
+  else
+    opencnn::wino_f32_fused<<<grid, block, 0, st>>>(a);
   return (int)hipGetLastError();
 }
 
@@ -129,6 +147,13 @@ size_t opencnn_workspace_bytes(int filt_c, int filt_k) {
 
 int opencnn_set_stream(void* stream) {
   g_stream.store(static_cast<hipStream_t>(stream));
+  return 0;
+}
+
+int opencnn_set_kernel_variant(int variant) {
+  REQUIRE(variant == OPENCNN_KERNEL_AUTO || variant == OPENCNN_KERNEL_REGISTER ||
+          variant == OPENCNN_KERNEL_LDS);
+  g_variant.store(variant);
   return 0;
 }
 

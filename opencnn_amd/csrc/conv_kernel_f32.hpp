@@ -88,6 +88,98 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, unsig
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, kBufferFlags);
 }
 
+// ------------------------------------------------------------------------------------------
+// Pieces shared by the kernels below.
+
+struct WaveTile {
+  int kg;        // 32-wide filter group
+  int ng;        // 32-wide batch group
+  int ty, tx;    // 2x2 output tile
+  int hsel, nl;  // lane = hsel*32 + nl: channel parity / batch element of this lane
+  int voff[16];  // byte offset of patch element (i,j) in a two-channel slab, or kOutOfRange
+};
+
+__device__ __forceinline__ void decode_tile(const ConvArgs& a, int kg, int cg, int lane, WaveTile& w) {
+  const int tile = cg / a.ngroups;
+  w.kg = kg;
+  w.ng = cg - tile * a.ngroups;
+  w.ty = tile / a.tiles_w;
+  w.tx = tile - w.ty * a.tiles_w;
+  w.hsel = lane >> 5;
+  w.nl = lane & 31;
+  const int HW = a.H * a.W;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int hh = 2 * w.ty - 1 + i, ww = 2 * w.tx - 1 + j;
+      const bool ok = hh >= 0 && hh < a.H && ww >= 0 && ww < a.W;
+      w.voff[i * 4 + j] =
+          ok ? (int)(((size_t)w.hsel * HW + (size_t)hh * a.W + ww) * a.N + w.ng * 32 + w.nl) * 4
+             : kOutOfRange;
+    }
+  }
+}
+
+// 4x4 patch of MFMA step `step` (channels 2*step + hsel); steps past the end reload the last
+// slab (the data is never used; this keeps the pipeline free of branches).
+__device__ __forceinline__ void load_patch(const ConvArgs& a, const WaveTile& w, float (&d)[16], int step) {
+  const int S = a.C >> 1;
+  const size_t HWN = (size_t)a.H * a.W * a.N;
+  const int st = step < S ? step : S - 1;
+  __amdgpu_buffer_rsrc_t r = make_rsrc(a.x + (size_t)st * 2 * HWN, (unsigned)(2 * HWN * sizeof(float)));
+#pragma unroll
+  for (int e = 0; e < 16; ++e)
+    d[e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, w.voff[e], 0, 0));
+}
+
+// A operands of filter quad `quad` (channels 4*quad .. 4*quad+3) for all 16 positions.
+__device__ __forceinline__ void load_u(const ConvArgs& a, const WaveTile& w, int lane, v2f (&u)[16], int quad) {
+  const int Q = a.C >> 2;
+  const __amdgpu_buffer_rsrc_t ru = make_rsrc(a.usw, (unsigned)((size_t)a.C * 16 * a.K * sizeof(float)));
+  const int qd = quad < Q ? quad : Q - 1;
+  const int soff = (w.kg * Q + qd) * (16 * 64 * 8);
+#pragma unroll
+  for (int p = 0; p < 16; ++p)
+    u[p] = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(ru, lane * 8 + p * 512, soff, 0));
+}
+
+// Output transform and store.  Accumulator register r of lane (hsel, nl) is row
+// k = 8*(r/4) + 4*hsel + r%4, column n = nl of the wave's 32x32 tile.
+__device__ __forceinline__ void store_tile(const ConvArgs& a, const WaveTile& w, const v16f (&acc)[16]) {
+  const size_t HWN = (size_t)a.H * a.W * a.N;
+  const bool row1 = 2 * w.ty + 1 < a.H;  // odd H: last tile row keeps only a = 0
+  const bool col1 = 2 * w.tx + 1 < a.W;  // odd W: last tile column keeps only b = 0
+  float* ybase = a.y + ((size_t)(2 * w.ty) * a.W + 2 * w.tx) * a.N + w.ng * 32 + w.nl;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    float m[16], o[4];
+#pragma unroll
+    for (int p = 0; p < 16; ++p) m[p] = acc[p][r];
+    output_transform(m, o);
+    const int k = w.kg * 32 + 8 * (r >> 2) + 4 * w.hsel + (r & 3);
+    float* yk = ybase + (size_t)k * HWN;
+    yk[0] = o[0];
+    if (col1) yk[a.N] = o[1];
+    if (row1) {
+      yk[(size_t)a.W * a.N] = o[2];
+      if (col1) yk[(size_t)a.W * a.N + a.N] = o[3];
+    }
+  }
+}
+
+// Logical block of this workgroup.  Workgroups are dealt round-robin to the 8 XCDs (one L2
+// each); every XCD gets a contiguous range of logical blocks so that blocks sharing input
+// columns and filters meet in one L2.
+__device__ __forceinline__ int logical_block() {
+  const int per_xcd = gridDim.x >> 3;
+  return (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+}
+
+// ------------------------------------------------------------------------------------------
+// Kernel A: every wave transforms its own patches (no LDS, no barriers).
+// Used when K is not a multiple of 64.
+//
 // One MFMA step = two input channels.  Software pipeline, per step t (all in registers):
 //   top     issue the 16 patch loads of step t+2 (and, every other step, the 16 filter
 //           loads of the quad after next);
@@ -98,58 +190,12 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, unsig
 __global__ void __launch_bounds__(256) wino_f32_fused(ConvArgs a) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-
-  // Workgroups are dealt round-robin to the 8 XCDs (one L2 each).  Give every XCD a
-  // contiguous range of logical blocks so that blocks sharing input columns (same
-  // column block, different k group) and filters (same k group) meet in one L2.
-  const int per_xcd = gridDim.x >> 3;
-  const int L = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  const int L = logical_block();
   if (L >= a.nblocks) return;
-  const int kg = L % a.kgroups;
   const int cg = (L / a.kgroups) * 4 + wave;
-  if (cg >= a.colgroups) return;  // wave-uniform; the kernel has no barriers
-
-  const int tile = cg / a.ngroups, ng = cg - tile * a.ngroups;
-  const int ty = tile / a.tiles_w, tx = tile - ty * a.tiles_w;
-  const int hsel = lane >> 5, nl = lane & 31;
-  const int HW = a.H * a.W;
-  const size_t HWN = (size_t)HW * a.N;
-
-  // Byte offset of patch element (i,j) inside a two-channel slab of x, or kOutOfRange.
-  int voff[16];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int hh = 2 * ty - 1 + i, ww = 2 * tx - 1 + j;
-      const bool ok = hh >= 0 && hh < a.H && ww >= 0 && ww < a.W;
-      voff[i * 4 + j] =
-          ok ? (int)(((size_t)hsel * HW + (size_t)hh * a.W + ww) * a.N + ng * 32 + nl) * 4
-             : kOutOfRange;
-    }
-  }
-  const unsigned slab_bytes = (unsigned)(2 * HWN * sizeof(float));
-  const int S = a.C >> 1;  // MFMA steps (two channels each)
-  const int Q = a.C >> 2;  // filter quads (two steps each)
-
-  auto load_patch = [&](float (&d)[16], int step) {
-    const int st = step < S ? step : S - 1;  // past the end: reload the last slab, unused
-    __amdgpu_buffer_rsrc_t r = make_rsrc(a.x + (size_t)st * 2 * HWN, slab_bytes);
-#pragma unroll
-    for (int e = 0; e < 16; ++e)
-      d[e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff[e], 0, 0));
-  };
-
-  const __amdgpu_buffer_rsrc_t ru =
-      make_rsrc(a.usw, (unsigned)((size_t)a.C * 16 * a.K * sizeof(float)));
-  const int uoff = lane * 8;
-  auto load_u = [&](v2f (&u)[16], int quad) {
-    const int qd = quad < Q ? quad : Q - 1;
-    const int soff = (kg * Q + qd) * (16 * 64 * 8);
-#pragma unroll
-    for (int p = 0; p < 16; ++p)
-      u[p] = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(ru, uoff + p * 512, soff, 0));
-  };
+  if (cg >= a.colgroups) return;  // wave-uniform; this kernel has no barriers
+  WaveTile w;
+  decode_tile(a, L % a.kgroups, cg, lane, w);
 
   v16f acc[16];
 #pragma unroll
@@ -162,9 +208,9 @@ __global__ void __launch_bounds__(256) wino_f32_fused(ConvArgs a) {
   float v[2][16];  // B operands: v[t&1] holds the transformed patch of step t
 
   // prologue: patch 0 -> v[0]; patch 1 in flight in d[1]; quad 0 in u[0]
-  load_u(u[0], 0);
-  load_patch(d[0], 0);
-  load_patch(d[1], 1);
+  load_u(a, w, lane, u[0], 0);
+  load_patch(a, w, d[0], 0);
+  load_patch(a, w, d[1], 1);
   input_transform(d[0], v[0]);
 
   const int octs = a.C >> 3;
@@ -173,9 +219,9 @@ __global__ void __launch_bounds__(256) wino_f32_fused(ConvArgs a) {
     for (int s = 0; s < 4; ++s) {
       const int t = oct * 4 + s;
       // d[t&1] was consumed by the transform of the previous step: refill it with step t+2
-      load_patch(d[s & 1], t + 2);
-      if (s == 0) load_u(u[1], 2 * oct + 1);
-      if (s == 2) load_u(u[0], 2 * oct + 2);
+      load_patch(a, w, d[s & 1], t + 2);
+      if (s == 0) load_u(a, w, lane, u[1], 2 * oct + 1);
+      if (s == 2) load_u(a, w, lane, u[0], 2 * oct + 2);
       __builtin_amdgcn_sched_barrier(0);
       input_transform(d[(s + 1) & 1], v[(s + 1) & 1]);
       // Anchor: the next B operands must exist when this region ends, or LLVM sinks the
@@ -193,27 +239,116 @@ __global__ void __launch_bounds__(256) wino_f32_fused(ConvArgs a) {
       __builtin_amdgcn_sched_barrier(0);
     }
   }
+  store_tile(a, w, acc);
+}
 
-  // Epilogue: accumulator register r of lane (hsel, nl) is row k = 8*(r/4) + 4*hsel + r%4,
-  // column n = nl of the 32x32 tile.
-  const bool row1 = 2 * ty + 1 < a.H;  // odd H: last tile row keeps only a = 0
-  const bool col1 = 2 * tx + 1 < a.W;  // odd W: last tile column keeps only b = 0
-  float* ybase = a.y + ((size_t)(2 * ty) * a.W + 2 * tx) * a.N + ng * 32 + nl;
+// ------------------------------------------------------------------------------------------
+// Kernel B: the KW waves of a workgroup that share one column tile (same spatial tile and
+// batch group, KW different filter groups) split the input transform between them and
+// exchange the transformed patches through LDS.
+//
+// Why: on gfx950 the fp32 MFMA and the fp32 VALU share the SIMD's ALUs (no co-execution:
+// every v_add/v_sub costs 4+ MFMA cycles), so the 32 add/sub per step of kernel A are paid in
+// full.  Sharing them KW ways cuts that to 32/KW; the LDS traffic that replaces them runs on
+// the LDS pipe in the shadow of the MFMAs.
+//
+// Workgroup = KW x CW waves (KW*CW = 4): wave = cw*KW + kw owns filter group kb*KW+kw and
+// column tile cb*CW+cw.  A chunk = 8 channels = 4 MFMA steps.  Wave kw transforms the steps
+// kw*SPW .. kw*SPW+SPW-1 (SPW = 4/KW) of every chunk for its column tile and writes them to
+//     V[cw][buf][step][p][lane]          (64 floats = one B operand register per wave)
+// in exactly the lane order in which all KW waves read them back as MFMA B operands, so
+// every LDS access is 256 contiguous bytes per wave: free of bank conflicts by construction.
+// Double buffered: chunk i reads buf i&1 while the transforms of chunk i+1 fill the other;
+// one workgroup barrier per chunk.
+template <int KW>
+__global__ void __launch_bounds__(256) wino_f32_fused_lds(ConvArgs a) {
+  constexpr int CW = 4 / KW;
+  constexpr int SPW = 4 / KW;
+  extern __shared__ float lds[];  // [CW][2][4][16][64]
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int kw = wave % KW, cw = wave / KW;
+  const int L = logical_block();
+  if (L >= a.nblocks) return;  // whole workgroup
+  const int kblocks = a.kgroups / KW;
+  const int cg_raw = (L / kblocks) * CW + cw;
+  const bool live = cg_raw < a.colgroups;
+  // A workgroup whose last column tile does not exist keeps those waves busy on a copy of
+  // the last real one (they must take part in the barriers) and drops their stores.
+  const int cg = live ? cg_raw : a.colgroups - 1;
+  WaveTile w;
+  decode_tile(a, (L % kblocks) * KW + kw, cg, lane, w);
+
+  float* vl = lds + cw * (2 * 4 * 16 * 64) + lane;
+  auto vaddr = [&](int buf, int step, int p) { return vl + ((buf * 4 + step) * 16 + p) * 64; };
+
+  v16f acc[16];
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    float m[16], o[4];
+  for (int p = 0; p < 16; ++p)
 #pragma unroll
-    for (int p = 0; p < 16; ++p) m[p] = acc[p][r];
-    output_transform(m, o);
-    const int k = kg * 32 + 8 * (r >> 2) + 4 * hsel + (r & 3);
-    float* yk = ybase + (size_t)k * HWN;
-    yk[0] = o[0];
-    if (col1) yk[a.N] = o[1];
-    if (row1) {
-      yk[(size_t)a.W * a.N] = o[2];
-      if (col1) yk[(size_t)a.W * a.N + a.N] = o[3];
+    for (int r = 0; r < 16; ++r) acc[p][r] = 0.0f;
+
+  v2f u[2][16];      // filter operands of the current / next quad
+  float d[SPW][16];  // this wave's share of the next chunk's patches, in flight
+  float v[2][16];    // B operands of the current / next step
+
+  auto transform_to_lds = [&](int buf) {
+#pragma unroll
+    for (int j = 0; j < SPW; ++j) {
+      float t[16];
+      input_transform(d[j], t);
+#pragma unroll
+      for (int p = 0; p < 16; ++p) *vaddr(buf, kw * SPW + j, p) = t[p];
     }
+  };
+  auto load_patches = [&](int chunk) {
+#pragma unroll
+    for (int j = 0; j < SPW; ++j) load_patch(a, w, d[j], chunk * 4 + kw * SPW + j);
+  };
+  auto read_v = [&](float (&dst)[16], int buf, int step) {
+#pragma unroll
+    for (int p = 0; p < 16; ++p) dst[p] = *vaddr(buf, step, p);
+  };
+  // LDS writes of this wave done, then workgroup barrier.  Deliberately not __syncthreads():
+  // that would also wait for the global loads in flight (vmcnt(0)) once per chunk.
+  auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+  // prologue: chunk 0 -> buf 0; chunk 1 patches in flight; quad 0 in u[0]
+  load_u(a, w, lane, u[0], 0);
+  load_patches(0);
+  transform_to_lds(0);
+  load_patches(1);
+  lds_barrier();
+  read_v(v[0], 0, 0);
+
+  const int chunks = a.C >> 3;
+  for (int i = 0; i < chunks; ++i) {
+    const int buf = i & 1;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      if (s == 0) load_u(a, w, lane, u[1], 2 * i + 1);
+      if (s == 2) load_u(a, w, lane, u[0], 2 * i + 2);
+      if (s < 3) read_v(v[(s + 1) & 1], buf, s + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      if (s == 0) transform_to_lds(buf ^ 1);  // chunk i+1
+#pragma unroll
+      for (int p = 0; p < 16; ++p)
+        acc[p] = __builtin_amdgcn_mfma_f32_32x32x2f32(u[s >> 1][p][s & 1], v[s & 1][p], acc[p], 0, 0, 0);
+      if (s == 0) {
+#pragma unroll
+        for (int p = 0; p < 16; ++p) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);            // one MFMA
+          __builtin_amdgcn_sched_group_barrier(0x002, 2 * SPW, 0);      // VALU of the transform
+          __builtin_amdgcn_sched_group_barrier(0x200, SPW, 0);          // its LDS writes
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (s == 0) load_patches(i + 2);
+    }
+    lds_barrier();
+    read_v(v[0], buf ^ 1, 0);
   }
+  if (live) store_tile(a, w, acc);
 }
 
 }  // namespace opencnn
