@@ -181,12 +181,13 @@ __device__ __forceinline__ int logical_block() {
 // Used when K is not a multiple of 64.
 //
 // One MFMA step = two input channels.  Software pipeline, per step t (all in registers):
-//   top     issue the 16 patch loads of step t+2 (and, every other step, the 16 filter
-//           loads of the quad after next);
-//   body    16 MFMAs of step t, interleaved with the 32 add/sub that turn the patch of
-//           step t+1 (loaded one step ago) into the next B operands.
-// The scheduling barriers keep hipcc from sinking the loads down to their first use (it
-// does so to save registers, which exposes the full memory latency once per step).
+//   first   the 32 add/sub that turn the patch of step t+1 (loaded one step ago) into the
+//           next B operands, as one burst (fp32 MFMA and fp32 VALU share the SIMD's ALUs on
+//           gfx950, and every MFMA->VALU->MFMA alternation costs extra cycles);
+//   then    the 16 MFMAs of step t, each followed by one or two of the loads of step t+2
+//           (16 patch loads and, every other step, the 16 filter loads of the next quad).
+// The scheduling barriers pin that order; left alone hipcc sinks the loads down to their
+// first use to save registers, which exposes the full memory latency once per step.
 __global__ void __launch_bounds__(256) wino_f32_fused(ConvArgs a) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -218,23 +219,29 @@ __global__ void __launch_bounds__(256) wino_f32_fused(ConvArgs a) {
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       const int t = oct * 4 + s;
-      // d[t&1] was consumed by the transform of the previous step: refill it with step t+2
-      load_patch(a, w, d[s & 1], t + 2);
-      if (s == 0) load_u(a, w, lane, u[1], 2 * oct + 1);
-      if (s == 2) load_u(a, w, lane, u[0], 2 * oct + 2);
       __builtin_amdgcn_sched_barrier(0);
       input_transform(d[(s + 1) & 1], v[(s + 1) & 1]);
       // Anchor: the next B operands must exist when this region ends, or LLVM sinks the
       // transform into the next step, in front of the MFMAs that need it.
 #pragma unroll
       for (int p = 0; p < 16; ++p) asm volatile("" : "+v"(v[(s + 1) & 1][p]));
+      __builtin_amdgcn_sched_barrier(0);
+      // d[t&1] was consumed by the transform of the previous step: refill it with step t+2
+      load_patch(a, w, d[s & 1], t + 2);
+      if (s == 0) load_u(a, w, lane, u[1], 2 * oct + 1);
+      if (s == 2) load_u(a, w, lane, u[0], 2 * oct + 2);
 #pragma unroll
       for (int p = 0; p < 16; ++p)
         acc[p] = __builtin_amdgcn_mfma_f32_32x32x2f32(u[s >> 1][p][s & 1], v[s & 1][p], acc[p], 0, 0, 0);
+      // Loads are spread behind the MFMAs (a burst of them stalls the wave on the vector
+      // memory address FIFO while the matrix pipe idles).
 #pragma unroll
       for (int p = 0; p < 16; ++p) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
-        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);  // two VALU of the next transform
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                        // one MFMA
+        if (s & 1)
+          __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one of the 16 patch loads
+        else
+          __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);  // patch load + filter load
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -326,24 +333,26 @@ __global__ void __launch_bounds__(256) wino_f32_fused_lds(ConvArgs a) {
     const int buf = i & 1;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
+      __builtin_amdgcn_sched_barrier(0);
+      if (s == 0) transform_to_lds(buf ^ 1);  // chunk i+1: one VALU burst, then its LDS writes
+      __builtin_amdgcn_sched_barrier(0);
       if (s == 0) load_u(a, w, lane, u[1], 2 * i + 1);
       if (s == 2) load_u(a, w, lane, u[0], 2 * i + 2);
+      if (s == 1) load_patches(i + 2);
       if (s < 3) read_v(v[(s + 1) & 1], buf, s + 1);
-      __builtin_amdgcn_sched_barrier(0);
-      if (s == 0) transform_to_lds(buf ^ 1);  // chunk i+1
 #pragma unroll
       for (int p = 0; p < 16; ++p)
         acc[p] = __builtin_amdgcn_mfma_f32_32x32x2f32(u[s >> 1][p][s & 1], v[s & 1][p], acc[p], 0, 0, 0);
-      if (s == 0) {
+      // One memory instruction behind every MFMA.  Issued as a burst, the loads fill the
+      // vector-memory address FIFO and the wave (the only one on its SIMD) sits on a load
+      // instead of feeding the matrix pipe; spread out, each is absorbed in an MFMA's shadow.
 #pragma unroll
-        for (int p = 0; p < 16; ++p) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);            // one MFMA
-          __builtin_amdgcn_sched_group_barrier(0x002, 2 * SPW, 0);      // VALU of the transform
-          __builtin_amdgcn_sched_group_barrier(0x200, SPW, 0);          // its LDS writes
-        }
+      for (int p = 0; p < 16; ++p) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // one MFMA
+        if (s != 3) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
+        if (s != 3 && (p & 1)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
       }
       __builtin_amdgcn_sched_barrier(0);
-      if (s == 0) load_patches(i + 2);
     }
     lds_barrier();
     read_v(v[0], buf ^ 1, 0);

@@ -212,6 +212,32 @@ def test_repeated_calls_are_identical_and_split_matches_dropin(ocn, torch_gpu):
     assert np.array_equal(y1, r.split())
 
 
+@pytest.mark.parametrize("variant", ["register", "lds"])
+@pytest.mark.parametrize("N,C,H,K", [(64, 64, 14, 64), (32, 24, 7, 128), (128, 128, 28, 128), (96, 8, 9, 256)])
+def test_both_kernel_variants(ocn, oracle, torch_gpu, variant, N, C, H, K):
+    # the register variant (every wave transforms its own patches) and the LDS variant (the
+    # waves of a workgroup share the transform) must both meet the bar on the same tensors
+    print(f"variant {variant} N={N} C={C} H={H} K={K}", flush=True)
+    x, w = make_tensors(ocn, N, C, H, H, K)
+    try:
+        ocn.set_kernel_variant(ocn.KERNEL_REGISTER if variant == "register" else ocn.KERNEL_LDS)
+        y = Runner(ocn, torch_gpu, x, w).dropin()
+    finally:
+        ocn.set_kernel_variant(ocn.KERNEL_AUTO)
+    check_against_oracle(oracle, y, x, w)
+
+
+def test_lds_variant_rejects_k_not_multiple_of_64(ocn, torch_gpu):
+    x, w = make_tensors(ocn, 32, 8, 6, 6, 96)
+    r = Runner(ocn, torch_gpu, x, w)
+    try:
+        ocn.set_kernel_variant(ocn.KERNEL_LDS)
+        with pytest.raises(ocn.OpenCNNError):
+            r.dropin()
+    finally:
+        ocn.set_kernel_variant(ocn.KERNEL_AUTO)
+
+
 def test_non_default_stream(ocn, oracle, torch_gpu):
     print("stream", flush=True)
     torch = torch_gpu
