@@ -112,6 +112,19 @@ enum { OPENCNN_KERNEL_AUTO = 0, OPENCNN_KERNEL_REGISTER = 1, OPENCNN_KERNEL_LDS 
 int opencnn_set_kernel_variant(int variant);
 
 /*
+ * Balanced split of the LDS kernel (default on).  When a layer has more workgroup tiles than
+ * the GPU has compute units, but not a whole number of rounds of them (784 tiles on 256 CUs =
+ * 3.06 rounds, which plain launching rounds up to 4), one persistent workgroup per CU takes an
+ * equal share of (tile, 8-channel chunk) units; a tile whose channel range ends up split
+ * between two workgroups is merged through the output tensor and two words of library-owned
+ * device state per wave.  Results stay independent of timing (two addends commute).  Calls
+ * that overlap in time on one GPU (different streams) must not both use it: pass 0 to turn it
+ * off.  No counterpart in the reference, whose grid is one block per tile
+ * (src/convolutionForward_32x64x8.cu:281).
+ */
+int opencnn_set_balanced_split(int enable);
+
+/*
  * The reference's FX kernel as a call of its own (src/FX_m2.cu:51-91, launched at
  * src/convolutionForward_32x64x8.cu:274): U = G g G^T for every (c,k).
  *   w              device, filt_c*9*filt_k floats in `filter_layout`

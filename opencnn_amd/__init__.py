@@ -18,6 +18,7 @@ from .binding import (  # noqa: F401
     load_library,
     set_stream,
     set_kernel_variant,
+    set_balanced_split,
     KERNEL_AUTO,
     KERNEL_REGISTER,
     KERNEL_LDS,

@@ -43,6 +43,7 @@ EXPORTED_SYMBOLS = {
     "opencnn_workspace_bytes": (ctypes.c_size_t, [_c_int, _c_int]),
     "opencnn_set_stream": (_c_int, [_c_void_p]),
     "opencnn_set_kernel_variant": (_c_int, [_c_int]),
+    "opencnn_set_balanced_split": (_c_int, [_c_int]),
     "opencnn_filter_transform": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int]),
     "opencnn_conv_forward_pretransformed": (
         _c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int]),
@@ -162,6 +163,12 @@ def set_stream(stream) -> None:
 def set_kernel_variant(variant: int) -> None:
     """KERNEL_AUTO, KERNEL_REGISTER or KERNEL_LDS for later launches."""
     _check("opencnn_set_kernel_variant", lib().opencnn_set_kernel_variant(variant))
+
+
+def set_balanced_split(enable: bool) -> None:
+    """Persistent, evenly split launch of the LDS kernel for tile counts that do not fill
+    whole rounds of CUs (default on)."""
+    _check("opencnn_set_balanced_split", lib().opencnn_set_balanced_split(1 if enable else 0))
 
 
 def convolutionForward(k, in_h, in_w, w, out_h, out_w, out_n, out_c, C, Ww, n, tiles_dim,

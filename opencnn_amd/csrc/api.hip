@@ -16,6 +16,23 @@ namespace {
 
 std::atomic<hipStream_t> g_stream{nullptr};
 std::atomic<int> g_variant{OPENCNN_KERNEL_AUTO};
+std::atomic<int> g_balance{1};
+
+// Compute units of the current device (cached per device index).
+int compute_units(int* out) {
+  static std::atomic<int> cache[64];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  int n = dev >= 0 && dev < 64 ? cache[dev].load() : 0;
+  if (n == 0) {
+    e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev >= 0 && dev < 64) cache[dev].store(n);
+  }
+  *out = n;
+  return 0;
+}
 thread_local const char* t_last_error = "";
 
 int fail(const char* what) {
@@ -102,17 +119,28 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   const int per_xcd = (a.nblocks + 7) / 8;
   dim3 grid(per_xcd * 8), block(256);
   const size_t lds_bytes = (size_t)cw * 2 * 4 * 16 * 64 * sizeof(float);
-  if (kw == 4)
-    opencnn::wino_f32_fused_lds<4><<<grid, block, lds_bytes, st>>>(a);
-  else if (kw == 2) {
-    // 96 KB of LDS: above the 64 KB a kernel gets without asking (gfx950 has 160 KB per CU)
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&opencnn::wino_f32_fused_lds<2>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-    if (e != hipSuccess) return (int)e;
-    opencnn::wino_f32_fused_lds<2><<<grid, block, lds_bytes, st>>>(a);
-  }
-  else
+  if (kw == 1) {
     opencnn::wino_f32_fused<<<grid, block, 0, st>>>(a);
+    return (int)hipGetLastError();
+  }
+  // More tiles than CUs and not a whole number of rounds: one persistent workgroup per CU,
+  // the chunk-units split evenly (every tile then has at most two contributors).
+  int cus = 0;
+  if (int e = compute_units(&cus)) return e;
+  const bool balanced = g_balance.load() != 0 && a.nblocks > cus && a.nblocks % cus != 0 &&
+                        cus % 8 == 0 && cus <= opencnn::kMaxBalancedBlocks;
+  if (balanced) grid = dim3(cus);
+  if (kw == 4) {
+    if (balanced)
+      opencnn::wino_f32_fused_lds<4, true><<<grid, block, lds_bytes, st>>>(a);
+    else
+      opencnn::wino_f32_fused_lds<4, false><<<grid, block, lds_bytes, st>>>(a);
+  } else {
+    if (balanced)
+      opencnn::wino_f32_fused_lds<2, true><<<grid, block, lds_bytes, st>>>(a);
+    else
+      opencnn::wino_f32_fused_lds<2, false><<<grid, block, lds_bytes, st>>>(a);
+  }
   return (int)hipGetLastError();
 }
 
@@ -154,6 +182,11 @@ int opencnn_set_kernel_variant(int variant) {
   REQUIRE(variant == OPENCNN_KERNEL_AUTO || variant == OPENCNN_KERNEL_REGISTER ||
           variant == OPENCNN_KERNEL_LDS);
   g_variant.store(variant);
+  return 0;
+}
+
+int opencnn_set_balanced_split(int enable) {
+  g_balance.store(enable != 0);
   return 0;
 }
 

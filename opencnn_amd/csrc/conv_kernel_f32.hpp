@@ -44,7 +44,7 @@ struct ConvArgs {
   int ngroups;           // N / 32
   int colgroups;         // tiles_h * tiles_w * ngroups   (wave-level column tiles)
   int kgroups;           // K / 32
-  int nblocks;           // ceil(colgroups / 4) * kgroups (4 waves = 4 column tiles per block)
+  int nblocks;           // workgroup tiles: column blocks x filter blocks
 };
 
 // V = B^T d B, columns first then rows (src/convolutionForward_32x64x8.cu:59-80).
@@ -146,11 +146,41 @@ __device__ __forceinline__ void load_u(const ConvArgs& a, const WaveTile& w, int
 
 // Output transform and store.  Accumulator register r of lane (hsel, nl) is row
 // k = 8*(r/4) + 4*hsel + r%4, column n = nl of the wave's 32x32 tile.
+//   kStorePlain    write the result
+//   kStorePublish  write a PARTIAL result (first half of a tile whose channel range is split
+//                  between two workgroups) straight through to memory, so that a wave on
+//                  another XCD (another L2) can read it without any cache-wide flush
+//   kStoreMerge    read the published partial result past the caches, add, write the result
+enum StoreMode { kStorePlain = 0, kStorePublish = 1, kStoreMerge = 2 };
+
+__device__ __forceinline__ float load_through(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+__device__ __forceinline__ void store_through(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+template <StoreMode MODE>
 __device__ __forceinline__ void store_tile(const ConvArgs& a, const WaveTile& w, const v16f (&acc)[16]) {
   const size_t HWN = (size_t)a.H * a.W * a.N;
   const bool row1 = 2 * w.ty + 1 < a.H;  // odd H: last tile row keeps only a = 0
   const bool col1 = 2 * w.tx + 1 < a.W;  // odd W: last tile column keeps only b = 0
   float* ybase = a.y + ((size_t)(2 * w.ty) * a.W + 2 * w.tx) * a.N + w.ng * 32 + w.nl;
+  const size_t o1 = a.N, o2 = (size_t)a.W * a.N, o3 = o2 + a.N;
+  // kStoreMerge: fetch the whole partial tile first (64 independent loads in flight at once;
+  // read one by one, each uncached load would cost a full trip to memory).
+  float part[MODE == kStoreMerge ? 16 : 1][4];
+  if (MODE == kStoreMerge) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int k = w.kg * 32 + 8 * (r >> 2) + 4 * w.hsel + (r & 3);
+      const float* yk = ybase + (size_t)k * HWN;
+      part[r][0] = load_through(yk);
+      part[r][1] = col1 ? load_through(yk + o1) : 0.0f;
+      part[r][2] = row1 ? load_through(yk + o2) : 0.0f;
+      part[r][3] = (row1 && col1) ? load_through(yk + o3) : 0.0f;
+    }
+  }
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     float m[16], o[4];
@@ -159,11 +189,24 @@ __device__ __forceinline__ void store_tile(const ConvArgs& a, const WaveTile& w,
     output_transform(m, o);
     const int k = w.kg * 32 + 8 * (r >> 2) + 4 * w.hsel + (r & 3);
     float* yk = ybase + (size_t)k * HWN;
-    yk[0] = o[0];
-    if (col1) yk[a.N] = o[1];
-    if (row1) {
-      yk[(size_t)a.W * a.N] = o[2];
-      if (col1) yk[(size_t)a.W * a.N + a.N] = o[3];
+    if (MODE == kStoreMerge) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) o[q] += part[r][q];
+    }
+    if (MODE == kStorePublish) {
+      store_through(yk, o[0]);
+      if (col1) store_through(yk + o1, o[1]);
+      if (row1) {
+        store_through(yk + o2, o[2]);
+        if (col1) store_through(yk + o3, o[3]);
+      }
+    } else {
+      yk[0] = o[0];
+      if (col1) yk[o1] = o[1];
+      if (row1) {
+        yk[o2] = o[2];
+        if (col1) yk[o3] = o[3];
+      }
     }
   }
 }
@@ -246,7 +289,7 @@ __global__ void __launch_bounds__(256) wino_f32_fused(ConvArgs a) {
       __builtin_amdgcn_sched_barrier(0);
     }
   }
-  store_tile(a, w, acc);
+  store_tile<kStorePlain>(a, w, acc);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -267,7 +310,22 @@ __global__ void __launch_bounds__(256) wino_f32_fused(ConvArgs a) {
 // every LDS access is 256 contiguous bytes per wave: free of bank conflicts by construction.
 // Double buffered: chunk i reads buf i&1 while the transforms of chunk i+1 fill the other;
 // one workgroup barrier per chunk.
-template <int KW>
+//
+// BALANCED = true turns the kernel into a persistent one: gridDim.x workgroups (one per CU)
+// share nblocks*chunks chunk-units evenly; a workgroup walks a contiguous range of units, so
+// its first and last tile may be covered only in part.  Without it 784 equal tiles on 256 CUs
+// take 4 rounds for 3.06 rounds of work.  The host only selects it when nblocks >= gridDim.x,
+// which bounds every tile to at most TWO contributing workgroups; their partial outputs are
+// merged through the output tensor itself: the wave that arrives first (atomic ticket) stores
+// its partial result and raises a flag, the second adds its own on top.  a+b == b+a in fp32,
+// so the result does not depend on the arrival order.  The second wave only ever waits for a
+// wave that is already running its epilogue, never for one that has yet to be scheduled.
+constexpr int kMaxBalancedBlocks = 1024;
+// [boundary between workgroups b and b+1][wave] -> {ticket, flag}; zero between launches
+// (the second contributor clears its pair).  Launches that overlap on one GPU would share it.
+static __device__ unsigned g_split_sync[kMaxBalancedBlocks * 4 * 2];
+
+template <int KW, bool BALANCED>
 __global__ void __launch_bounds__(256) wino_f32_fused_lds(ConvArgs a) {
   constexpr int CW = 4 / KW;
   constexpr int SPW = 4 / KW;
@@ -276,88 +334,139 @@ __global__ void __launch_bounds__(256) wino_f32_fused_lds(ConvArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int kw = wave % KW, cw = wave / KW;
   const int L = logical_block();
-  if (L >= a.nblocks) return;  // whole workgroup
   const int kblocks = a.kgroups / KW;
-  const int cg_raw = (L / kblocks) * CW + cw;
-  const bool live = cg_raw < a.colgroups;
-  // A workgroup whose last column tile does not exist keeps those waves busy on a copy of
-  // the last real one (they must take part in the barriers) and drops their stores.
-  const int cg = live ? cg_raw : a.colgroups - 1;
-  WaveTile w;
-  decode_tile(a, (L % kblocks) * KW + kw, cg, lane, w);
+  const int chunks = a.C >> 3;
+
+  // chunk-units [unit, end) of this workgroup; unit = tile * chunks + chunk
+  long long unit, end;
+  if (BALANCED) {
+    const long long total = (long long)a.nblocks * chunks;
+    unit = total * L / gridDim.x;
+    end = total * (L + 1) / gridDim.x;
+  } else {
+    if (L >= a.nblocks) return;  // whole workgroup
+    unit = (long long)L * chunks;
+    end = unit + chunks;
+  }
 
   float* vl = lds + cw * (2 * 4 * 16 * 64) + lane;
   auto vaddr = [&](int buf, int step, int p) { return vl + ((buf * 4 + step) * 16 + p) * 64; };
-
-  v16f acc[16];
-#pragma unroll
-  for (int p = 0; p < 16; ++p)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc[p][r] = 0.0f;
-
-  v2f u[2][16];      // filter operands of the current / next quad
-  float d[SPW][16];  // this wave's share of the next chunk's patches, in flight
-  float v[2][16];    // B operands of the current / next step
-
-  auto transform_to_lds = [&](int buf) {
-#pragma unroll
-    for (int j = 0; j < SPW; ++j) {
-      float t[16];
-      input_transform(d[j], t);
-#pragma unroll
-      for (int p = 0; p < 16; ++p) *vaddr(buf, kw * SPW + j, p) = t[p];
-    }
-  };
-  auto load_patches = [&](int chunk) {
-#pragma unroll
-    for (int j = 0; j < SPW; ++j) load_patch(a, w, d[j], chunk * 4 + kw * SPW + j);
-  };
-  auto read_v = [&](float (&dst)[16], int buf, int step) {
-#pragma unroll
-    for (int p = 0; p < 16; ++p) dst[p] = *vaddr(buf, step, p);
-  };
   // LDS writes of this wave done, then workgroup barrier.  Deliberately not __syncthreads():
   // that would also wait for the global loads in flight (vmcnt(0)) once per chunk.
   auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
-  // prologue: chunk 0 -> buf 0; chunk 1 patches in flight; quad 0 in u[0]
-  load_u(a, w, lane, u[0], 0);
-  load_patches(0);
-  transform_to_lds(0);
-  load_patches(1);
-  lds_barrier();
-  read_v(v[0], 0, 0);
+  while (unit < end) {
+    const int T = (int)(unit / chunks);
+    const int c0 = (int)(unit - (long long)T * chunks);
+    const int c1 = (end - unit) < (long long)(chunks - c0) ? c0 + (int)(end - unit) : chunks;
+    unit += c1 - c0;
 
-  const int chunks = a.C >> 3;
-  for (int i = 0; i < chunks; ++i) {
-    const int buf = i & 1;
+    const int cg_raw = (T / kblocks) * CW + cw;
+    const bool live = cg_raw < a.colgroups;
+    // A workgroup whose last column tile does not exist keeps those waves busy on a copy of
+    // the last real one (they must take part in the barriers) and drops their stores.
+    const int cg = live ? cg_raw : a.colgroups - 1;
+    WaveTile w;
+    decode_tile(a, (T % kblocks) * KW + kw, cg, lane, w);
+
+    v16f acc[16];
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      __builtin_amdgcn_sched_barrier(0);
-      if (s == 0) transform_to_lds(buf ^ 1);  // chunk i+1: one VALU burst, then its LDS writes
-      __builtin_amdgcn_sched_barrier(0);
-      if (s == 0) load_u(a, w, lane, u[1], 2 * i + 1);
-      if (s == 2) load_u(a, w, lane, u[0], 2 * i + 2);
-      if (s == 1) load_patches(i + 2);
-      if (s < 3) read_v(v[(s + 1) & 1], buf, s + 1);
+    for (int p = 0; p < 16; ++p)
 #pragma unroll
-      for (int p = 0; p < 16; ++p)
-        acc[p] = __builtin_amdgcn_mfma_f32_32x32x2f32(u[s >> 1][p][s & 1], v[s & 1][p], acc[p], 0, 0, 0);
-      // One memory instruction behind every MFMA.  Issued as a burst, the loads fill the
-      // vector-memory address FIFO and the wave (the only one on its SIMD) sits on a load
-      // instead of feeding the matrix pipe; spread out, each is absorbed in an MFMA's shadow.
+      for (int r = 0; r < 16; ++r) acc[p][r] = 0.0f;
+
+    v2f u[2][16];      // filter operands of the current / next quad
+    float d[SPW][16];  // this wave's share of the next chunk's patches, in flight
+    float v[2][16];    // B operands of the current / next step
+
+    auto transform_to_lds = [&](int buf) {
 #pragma unroll
-      for (int p = 0; p < 16; ++p) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // one MFMA
-        if (s != 3) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
-        if (s != 3 && (p & 1)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+      for (int j = 0; j < SPW; ++j) {
+        float t[16];
+        input_transform(d[j], t);
+#pragma unroll
+        for (int p = 0; p < 16; ++p) *vaddr(buf, kw * SPW + j, p) = t[p];
       }
-      __builtin_amdgcn_sched_barrier(0);
-    }
+    };
+    auto load_patches = [&](int chunk) {
+#pragma unroll
+      for (int j = 0; j < SPW; ++j) load_patch(a, w, d[j], chunk * 4 + kw * SPW + j);
+    };
+    auto read_v = [&](float (&dst)[16], int buf, int step) {
+#pragma unroll
+      for (int p = 0; p < 16; ++p) dst[p] = *vaddr(buf, step, p);
+    };
+
+    // prologue: chunk c0 -> buf 0; chunk c0+1 patches in flight; first quad in u[0].
+    // (All reads of the previous tile's LDS data precede its last barrier, so buf 0 is free.)
+    load_u(a, w, lane, u[0], 2 * c0);
+    load_patches(c0);
+    transform_to_lds(0);
+    load_patches(c0 + 1);
     lds_barrier();
-    read_v(v[0], buf ^ 1, 0);
+    read_v(v[0], 0, 0);
+
+    for (int i = c0; i < c1; ++i) {
+      const int buf = (i - c0) & 1;
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (s == 0) transform_to_lds(buf ^ 1);  // chunk i+1: one VALU burst, then its LDS writes
+        __builtin_amdgcn_sched_barrier(0);
+        if (s == 0) load_u(a, w, lane, u[1], 2 * i + 1);
+        if (s == 2) load_u(a, w, lane, u[0], 2 * i + 2);
+        if (s == 1) load_patches(i + 2);
+        if (s < 3) read_v(v[(s + 1) & 1], buf, s + 1);
+#pragma unroll
+        for (int p = 0; p < 16; ++p)
+          acc[p] = __builtin_amdgcn_mfma_f32_32x32x2f32(u[s >> 1][p][s & 1], v[s & 1][p], acc[p], 0, 0, 0);
+        // One memory instruction behind every MFMA.  Issued as a burst, the loads fill the
+        // vector-memory address FIFO and the wave (the only one on its SIMD) sits on a load
+        // instead of feeding the matrix pipe; spread out, each is absorbed in an MFMA's shadow.
+#pragma unroll
+        for (int p = 0; p < 16; ++p) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // one MFMA
+          if (s != 3) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
+          if (s != 3 && (p & 1)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      lds_barrier();
+      read_v(v[0], buf ^ 1, 0);
+    }
+
+    if (!live) continue;
+    if (!BALANCED || (c0 == 0 && c1 == chunks)) {
+      store_tile<kStorePlain>(a, w, acc);
+      continue;
+    }
+    // Partial tile: the other part belongs to the previous (c0 > 0) or next workgroup.
+    // All traffic of the hand-over (partial result, ticket, flag) goes straight to memory with
+    // per-access system-scope policy; no fence is used, because a device-scope fence writes
+    // back / invalidates the whole L2 of the XCD under the other 31 workgroups' feet.
+    unsigned* sync = g_split_sync + ((c0 > 0 ? L - 1 : L) * 4 + wave) * 2;
+    unsigned ticket = 0;
+    if (lane == 0) ticket = __hip_atomic_fetch_add(sync, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    ticket = __builtin_amdgcn_readfirstlane(ticket);
+    if (ticket == 0) {
+      store_tile<kStorePublish>(a, w, acc);
+      // every write-through store of this wave acknowledged, then raise the flag
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (lane == 0) __hip_atomic_store(sync + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    } else {
+      // The first contributor holds ticket 0 and is in its epilogue; bounded wait all the same.
+      for (int spin = 0; spin < (1 << 22); ++spin) {
+        if (__hip_atomic_load(sync + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0) break;
+        __builtin_amdgcn_s_sleep(8);
+      }
+      asm volatile("" ::: "memory");  // the partial result is read after the flag, not before
+      store_tile<kStoreMerge>(a, w, acc);
+      if (lane == 0) {
+        __hip_atomic_store(sync, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        __hip_atomic_store(sync + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      }
+    }
   }
-  if (live) store_tile(a, w, acc);
 }
 
 }  // namespace opencnn

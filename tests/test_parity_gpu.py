@@ -238,6 +238,28 @@ def test_lds_variant_rejects_k_not_multiple_of_64(ocn, torch_gpu):
         ocn.set_kernel_variant(ocn.KERNEL_AUTO)
 
 
+@pytest.mark.parametrize("N,C,H,K", [(64, 16, 40, 128), (32, 64, 45, 64), (96, 8, 33, 128)])
+def test_balanced_split_matches_plain_launch(ocn, oracle, torch_gpu, N, C, H, K):
+    # more workgroup tiles than CUs and not a whole number of rounds: the persistent,
+    # evenly split launch merges tiles cut between two workgroups.  It must meet the bar,
+    # repeat bit for bit (the merge is a two-term sum), and stay within rounding of the
+    # plain one-tile-per-workgroup launch.
+    print(f"balanced N={N} C={C} H={H} K={K}", flush=True)
+    x, w = make_tensors(ocn, N, C, H, H, K)
+    r = Runner(ocn, torch_gpu, x, w)
+    y1 = r.dropin()
+    y2 = r.dropin()
+    assert np.array_equal(y1, y2)
+    check_against_oracle(oracle, y1, x, w)
+    try:
+        ocn.set_balanced_split(False)
+        y0 = r.dropin()
+    finally:
+        ocn.set_balanced_split(True)
+    check_against_oracle(oracle, y0, x, w)
+    np.testing.assert_allclose(y1, y0, rtol=0, atol=2e-6 * np.abs(y0).max())
+
+
 def test_non_default_stream(ocn, oracle, torch_gpu):
     print("stream", flush=True)
     torch = torch_gpu
