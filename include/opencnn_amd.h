@@ -40,8 +40,17 @@ enum {
   OPENCNN_FILTER_KCRS = 1  /* the cuDNN-side layout of the reference's bench (src/openCNN_winograd.cu:234) */
 };
 
-/* GEMM operand precision of the fused kernel (transforms and accumulation stay fp32). */
+/*
+ * GEMM operand precision of later calls (default OPENCNN_F32, the reference's only mode).
+ * With OPENCNN_F16 / OPENCNN_BF16 both transforms and the accumulation stay fp32, but the
+ * transformed input and the transformed filter are rounded to nearest-even once and the 16
+ * batched GEMMs run on fp16 / bf16 MFMA.  Ww then holds 2-byte elements (half of the buffer
+ * is used).  Needs in_c % 16 == 0 and filt_k % 64 == 0.  Tensors in HBM stay fp32.
+ * opencnn_filter_transform(..., OPENCNN_WW_MFMA) and the fused kernel must run under the same
+ * setting.
+ */
 enum { OPENCNN_F32 = 0, OPENCNN_F16 = 1, OPENCNN_BF16 = 2 };
+int opencnn_set_operand_precision(int precision);
 
 /*
  * Replaces the reference's hidden set-up: the caller-side cudaMemcpyToSymbol uploads of

@@ -19,6 +19,10 @@ from .binding import (  # noqa: F401
     set_stream,
     set_kernel_variant,
     set_balanced_split,
+    set_operand_precision,
+    F32,
+    F16,
+    BF16,
     KERNEL_AUTO,
     KERNEL_REGISTER,
     KERNEL_LDS,

@@ -21,6 +21,7 @@ FILTER_CRSK, FILTER_KCRS = 0, 1
 INPUT_CHWN, INPUT_NCHW = 0, 1
 DIST_UNIFORM, DIST_NORMAL = 0, 1
 KERNEL_AUTO, KERNEL_REGISTER, KERNEL_LDS = 0, 1, 2
+F32, F16, BF16 = 0, 1, 2
 
 _c_int, _c_float_p, _c_void_p = ctypes.c_int, ctypes.POINTER(ctypes.c_float), ctypes.c_void_p
 
@@ -44,6 +45,7 @@ EXPORTED_SYMBOLS = {
     "opencnn_set_stream": (_c_int, [_c_void_p]),
     "opencnn_set_kernel_variant": (_c_int, [_c_int]),
     "opencnn_set_balanced_split": (_c_int, [_c_int]),
+    "opencnn_set_operand_precision": (_c_int, [_c_int]),
     "opencnn_filter_transform": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int]),
     "opencnn_conv_forward_pretransformed": (
         _c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int]),
@@ -169,6 +171,11 @@ def set_balanced_split(enable: bool) -> None:
     """Persistent, evenly split launch of the LDS kernel for tile counts that do not fill
     whole rounds of CUs (default on)."""
     _check("opencnn_set_balanced_split", lib().opencnn_set_balanced_split(1 if enable else 0))
+
+
+def set_operand_precision(precision: int) -> None:
+    """F32 (default), F16 or BF16 GEMM operands for later calls."""
+    _check("opencnn_set_operand_precision", lib().opencnn_set_operand_precision(precision))
 
 
 def convolutionForward(k, in_h, in_w, w, out_h, out_w, out_n, out_c, C, Ww, n, tiles_dim,

@@ -10,6 +10,7 @@
 #include <cstring>
 
 #include "conv_kernel_f32.hpp"
+#include "conv_kernel_h16.hpp"
 #include "fx_kernels.hpp"
 
 namespace {
@@ -17,6 +18,7 @@ namespace {
 std::atomic<hipStream_t> g_stream{nullptr};
 std::atomic<int> g_variant{OPENCNN_KERNEL_AUTO};
 std::atomic<int> g_balance{1};
+std::atomic<int> g_precision{OPENCNN_F32};
 
 // Compute units of the current device (cached per device index).
 int compute_units(int* out) {
@@ -72,6 +74,24 @@ int launch_fx(const float* w, float* Ww, int filt_k, int filt_c, int filter_layo
   REQUIRE(ww_layout == OPENCNN_WW_REFERENCE || ww_layout == OPENCNN_WW_MFMA);
   if (int e = check_filter_shape(filt_k, filt_c)) return e;
   const bool kcrs = filter_layout == OPENCNN_FILTER_KCRS;
+  const int precision = g_precision.load();
+  if (ww_layout == OPENCNN_WW_MFMA && precision != OPENCNN_F32) {
+    REQUIRE(filt_c % 16 == 0);
+    dim3 grid((filt_k + 127) / 128, filt_c / 16), block(256);
+    uint4* out = reinterpret_cast<uint4*>(Ww);
+    if (precision == OPENCNN_F16) {
+      if (kcrs)
+        opencnn::fx_mfma_layout_h16<true, false><<<grid, block, 0, st>>>(w, out, filt_k, filt_c);
+      else
+        opencnn::fx_mfma_layout_h16<false, false><<<grid, block, 0, st>>>(w, out, filt_k, filt_c);
+    } else {
+      if (kcrs)
+        opencnn::fx_mfma_layout_h16<true, true><<<grid, block, 0, st>>>(w, out, filt_k, filt_c);
+      else
+        opencnn::fx_mfma_layout_h16<false, true><<<grid, block, 0, st>>>(w, out, filt_k, filt_c);
+    }
+    return (int)hipGetLastError();
+  }
   if (ww_layout == OPENCNN_WW_REFERENCE) {
     dim3 grid((filt_k + 255) / 256, filt_c), block(256);
     if (kcrs)
@@ -106,6 +126,37 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   a.ngroups = in_n / 32;
   a.colgroups = a.tiles_h * a.tiles_w * a.ngroups;
   a.kgroups = filt_k / 32;
+  const int precision = g_precision.load();
+  if (precision != OPENCNN_F32) {
+    // fp16 / bf16 GEMM operands: 16-channel chunks, LDS kernel only
+    REQUIRE(in_c % 16 == 0);
+    REQUIRE(filt_k % 64 == 0);
+    REQUIRE((long long)in_n * in_h * in_w * 4 * 4 <= kMaxElems);  // four-channel window in bytes
+    const int hkw = filt_k % 128 == 0 ? 4 : 2, hcw = 4 / hkw;
+    const long long hblocks = (long long)((a.colgroups + hcw - 1) / hcw) * (a.kgroups / hkw);
+    REQUIRE(hblocks <= kMaxElems / 8);
+    a.nblocks = (int)hblocks;
+    dim3 hgrid(((a.nblocks + 7) / 8) * 8), hblock(256);
+    const size_t hlds = (size_t)hcw * 3 * 16 * 2 * 4 * 32 * sizeof(unsigned);
+    const bool bf = precision == OPENCNN_BF16;
+    if (hkw == 4) {
+      if (bf)
+        opencnn::wino_h16_fused_lds<4, true><<<hgrid, hblock, hlds, st>>>(a);
+      else
+        opencnn::wino_h16_fused_lds<4, false><<<hgrid, hblock, hlds, st>>>(a);
+    } else {
+      // 96 KB of LDS: above the 64 KB a kernel gets without asking (gfx950 has 160 KB per CU)
+      const void* fn = bf ? reinterpret_cast<const void*>(&opencnn::wino_h16_fused_lds<2, true>)
+                          : reinterpret_cast<const void*>(&opencnn::wino_h16_fused_lds<2, false>);
+      hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)hlds);
+      if (e != hipSuccess) return (int)e;
+      if (bf)
+        opencnn::wino_h16_fused_lds<2, true><<<hgrid, hblock, hlds, st>>>(a);
+      else
+        opencnn::wino_h16_fused_lds<2, false><<<hgrid, hblock, hlds, st>>>(a);
+    }
+    return (int)hipGetLastError();
+  }
   // Waves per workgroup that share one column tile (and split its input transform).
   int kw = 1;
   const int variant = g_variant.load();
@@ -182,6 +233,12 @@ int opencnn_set_kernel_variant(int variant) {
   REQUIRE(variant == OPENCNN_KERNEL_AUTO || variant == OPENCNN_KERNEL_REGISTER ||
           variant == OPENCNN_KERNEL_LDS);
   g_variant.store(variant);
+  return 0;
+}
+
+int opencnn_set_operand_precision(int precision) {
+  REQUIRE(precision == OPENCNN_F32 || precision == OPENCNN_F16 || precision == OPENCNN_BF16);
+  g_precision.store(precision);
   return 0;
 }
 

@@ -86,4 +86,43 @@ __global__ void __launch_bounds__(256) fx_mfma_layout(const float* __restrict__ 
   for (int p = 0; p < 16; ++p) o[(size_t)p * 64] = make_float2(U0[p], U1[p]);
 }
 
+// Reduced-precision MFMA-operand layout read by the fp16 / bf16 fused kernel:
+//   Uh[kg][chunk][p][h][k32][e] (2-byte elements),  k = kg*32 + k32,  c = 16*chunk + 8*h + e
+// so that lane (h*32 + k32) of a wave fetches, with one 16-byte load per position p, the A
+// operand of one v_mfma_f32_32x32x16_{f16,bf16} (16 input channels).  U is computed in fp32 in
+// the reference's order and rounded to nearest-even once.  Thread = (k, chunk, h).
+// grid (ceil(K/128), C/16), block 256 = 2 h x 128 k.
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+typedef __bf16 v2b __attribute__((ext_vector_type(2)));
+typedef float v2fx __attribute__((ext_vector_type(2)));
+
+template <bool BF16>
+__device__ __forceinline__ unsigned pack_pair(float lo, float hi) {
+  v2fx f = {lo, hi};
+  if (BF16) return __builtin_bit_cast(unsigned, __builtin_convertvector(f, v2b));
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(f, v2h));
+}
+
+template <bool KCRS, bool BF16>
+__global__ void __launch_bounds__(256) fx_mfma_layout_h16(const float* __restrict__ w,
+                                                          uint4* __restrict__ Uh, int K, int C) {
+  const int h = threadIdx.x >> 7;
+  const int k = blockIdx.x * 128 + (threadIdx.x & 127);
+  const int chunk = blockIdx.y;
+  if (k >= K) return;
+  float U[8][16];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    float g[9];
+    load_filter<KCRS>(w, 16 * chunk + 8 * h + e, k, C, K, g);
+    fx_one(g, U[e]);
+  }
+  const int kg = k >> 5, k32 = k & 31;
+  uint4* o = Uh + (((size_t)kg * (C >> 4) + chunk) * 16) * 64 + h * 32 + k32;
+#pragma unroll
+  for (int p = 0; p < 16; ++p)
+    o[(size_t)p * 64] = make_uint4(pack_pair<BF16>(U[0][p], U[1][p]), pack_pair<BF16>(U[2][p], U[3][p]),
+                                   pack_pair<BF16>(U[4][p], U[5][p]), pack_pair<BF16>(U[6][p], U[7][p]));
+}
+
 }  // namespace opencnn

@@ -260,6 +260,53 @@ def test_balanced_split_matches_plain_launch(ocn, oracle, torch_gpu, N, C, H, K)
     np.testing.assert_allclose(y1, y0, rtol=0, atol=2e-6 * np.abs(y0).max())
 
 
+# ---------------------------------------------------------------- fp16 / bf16 GEMM operands
+
+# bounds against the fp64 direct convolution: unit round-offs 2^-11 (fp16) and 2^-8 (bf16) on
+# both GEMM operands; against the oracle's quantised restatement (same roundings, fp32 chain)
+# only the summation order differs
+REL_L2_DIRECT_REDUCED = {"f16": 2e-3, "bf16": 1.5e-2}
+REL_L2_QUANTISED_RESTATEMENT = 2e-5
+
+
+@pytest.mark.parametrize("prec", ["f16", "bf16"])
+@pytest.mark.parametrize("N,C,H,K,xr", [
+    (128, 256, 14, 256, (-1.0, 1.0)),  # the reduced-precision benchmark configuration
+    (32, 16, 7, 64, (-1.0, 1.0)),      # odd size, two waves per column tile
+    (64, 48, 9, 128, (0.0, 1.0)),      # odd number of 16-channel chunks
+    (32, 32, 4, 192, (-1.0, 1.0)),
+])
+def test_reduced_precision_operands(ocn, oracle, torch_gpu, prec, N, C, H, K, xr):
+    print(f"reduced {prec} N={N} C={C} H={H} K={K}", flush=True)
+    x, w = make_tensors(ocn, N, C, H, H, K, xr)
+    quant = 1 if prec == "f16" else 2
+    try:
+        ocn.set_operand_precision(ocn.F16 if prec == "f16" else ocn.BF16)
+        r = Runner(ocn, torch_gpu, x, w)
+        y = r.dropin()
+        y2 = r.dropin()
+    finally:
+        ocn.set_operand_precision(ocn.F32)
+    assert not np.isnan(y).any()
+    assert np.array_equal(y, y2)
+    rel, max_abs, max_ref = oracle.compare(y, oracle.winograd_f32(x, w, quant))
+    assert rel <= REL_L2_QUANTISED_RESTATEMENT, f"rel-L2 vs quantised restatement {rel:.3e}"
+    rel64, _, _ = oracle.compare(y, oracle.direct_conv_f64(x, w))
+    assert 1e-5 < rel64 <= REL_L2_DIRECT_REDUCED[prec], f"rel-L2 vs fp64 direct {rel64:.3e}"
+    print(f"  rel-L2 vs quantised restatement {rel:.2e}, vs fp64 direct {rel64:.2e}", flush=True)
+
+
+def test_reduced_precision_rejects_unsupported_shapes(ocn, torch_gpu):
+    x, w = make_tensors(ocn, 32, 8, 6, 6, 64)  # C % 16 != 0
+    r = Runner(ocn, torch_gpu, x, w)
+    try:
+        ocn.set_operand_precision(ocn.F16)
+        with pytest.raises(ocn.OpenCNNError):
+            r.dropin()
+    finally:
+        ocn.set_operand_precision(ocn.F32)
+
+
 def test_non_default_stream(ocn, oracle, torch_gpu):
     print("stream", flush=True)
     torch = torch_gpu
