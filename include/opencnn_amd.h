@@ -167,6 +167,17 @@ int opencnn_time_forward(const float *in, const float *w, float *out, float *Ww,
                          int in_n, int in_c, int in_h, int in_w, int filt_k, int warmup,
                          int iters, float *ms_total, float *ms_main, float *ms_fx);
 
+/*
+ * Layout shims on the selected stream, device to device, src != dst: the reference's data_cpy
+ * kernel (src/openCNN_winograd.cu:147-153) as used at :230 (NCHW input -> CHWN) and :235 (KCRS
+ * filters -> CRSK), plus the way back for the result (KHWN -> NKHW, i.e. NCHW with K channels),
+ * which the reference only does implicitly inside its checker's index map (:185-186).
+ * data_cpy is limited to C <= 1024 by its launch shape; these are not.
+ */
+int opencnn_nchw_to_chwn(const float *src, float *dst, int n, int c, int h, int w);
+int opencnn_khwn_to_nkhw(const float *src, float *dst, int n, int k, int h, int w);
+int opencnn_kcrs_to_crsk(const float *src, float *dst, int k, int c);
+
 /* Layout of a synthetic input written by opencnn_synth_input. */
 enum { OPENCNN_INPUT_CHWN = 0, OPENCNN_INPUT_NCHW = 1 };
 /* Distribution of a synthetic tensor: uniform on [p0,p1) or normal(mean p0, std p1). */

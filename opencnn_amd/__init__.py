@@ -19,6 +19,9 @@ from .binding import (  # noqa: F401
     set_stream,
     set_kernel_variant,
     set_balanced_split,
+    nchw_to_chwn,
+    khwn_to_nkhw,
+    kcrs_to_crsk,
     set_operand_precision,
     F32,
     F16,

@@ -49,6 +49,9 @@ EXPORTED_SYMBOLS = {
     "opencnn_filter_transform": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int]),
     "opencnn_conv_forward_pretransformed": (
         _c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int]),
+    "opencnn_nchw_to_chwn": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int]),
+    "opencnn_khwn_to_nkhw": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int]),
+    "opencnn_kcrs_to_crsk": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int]),
     "opencnn_time_forward": (
         _c_int,
         [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -200,6 +203,18 @@ def conv_forward_pretransformed(x, Ww, y, in_n, in_c, in_h, in_w, filt_k) -> Non
     _check("opencnn_conv_forward_pretransformed", lib().opencnn_conv_forward_pretransformed(
         _dev_f32(x, "input"), _dev_f32(Ww, "workspace"), _dev_f32(y, "output"), in_n, in_c,
         in_h, in_w, filt_k))
+
+
+def nchw_to_chwn(src, dst, n, c, h, w) -> None:
+    _check("opencnn_nchw_to_chwn", lib().opencnn_nchw_to_chwn(_dev_f32(src, "src"), _dev_f32(dst, "dst"), n, c, h, w))
+
+
+def khwn_to_nkhw(src, dst, n, k, h, w) -> None:
+    _check("opencnn_khwn_to_nkhw", lib().opencnn_khwn_to_nkhw(_dev_f32(src, "src"), _dev_f32(dst, "dst"), n, k, h, w))
+
+
+def kcrs_to_crsk(src, dst, k, c) -> None:
+    _check("opencnn_kcrs_to_crsk", lib().opencnn_kcrs_to_crsk(_dev_f32(src, "src"), _dev_f32(dst, "dst"), k, c))
 
 
 def time_forward(x, w, y, Ww, in_n, in_c, in_h, in_w, filt_k, warmup=1, iters=100):

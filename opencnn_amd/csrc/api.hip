@@ -12,6 +12,7 @@
 #include "conv_kernel_f32.hpp"
 #include "conv_kernel_h16.hpp"
 #include "fx_kernels.hpp"
+#include "layout_kernels.hpp"
 
 namespace {
 
@@ -105,6 +106,15 @@ int launch_fx(const float* w, float* Ww, int filt_k, int filt_c, int filter_layo
     else
       opencnn::fx_mfma_layout<false><<<grid, block, 0, st>>>(w, Ww, filt_k, filt_c);
   }
+  return (int)hipGetLastError();
+}
+
+int launch_transpose(const float* src, float* dst, long long rows, long long cols, hipStream_t st) {
+  REQUIRE(src != nullptr && dst != nullptr && src != dst);
+  REQUIRE(rows > 0 && cols > 0 && rows * cols <= kMaxElems);
+  REQUIRE((rows + 63) / 64 <= 65535);  // gridDim.y
+  dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64)), block(256);
+  opencnn::transpose_2d<<<grid, block, 0, st>>>(src, dst, (int)rows, (int)cols);
   return (int)hipGetLastError();
 }
 
@@ -234,6 +244,21 @@ int opencnn_set_kernel_variant(int variant) {
           variant == OPENCNN_KERNEL_LDS);
   g_variant.store(variant);
   return 0;
+}
+
+int opencnn_nchw_to_chwn(const float* src, float* dst, int n, int c, int h, int w) {
+  REQUIRE(n > 0 && c > 0 && h > 0 && w > 0);
+  return launch_transpose(src, dst, n, (long long)c * h * w, g_stream.load());
+}
+
+int opencnn_khwn_to_nkhw(const float* src, float* dst, int n, int k, int h, int w) {
+  REQUIRE(n > 0 && k > 0 && h > 0 && w > 0);
+  return launch_transpose(src, dst, (long long)k * h * w, n, g_stream.load());
+}
+
+int opencnn_kcrs_to_crsk(const float* src, float* dst, int k, int c) {
+  REQUIRE(k > 0 && c > 0);
+  return launch_transpose(src, dst, k, (long long)c * 9, g_stream.load());
 }
 
 int opencnn_set_operand_precision(int precision) {

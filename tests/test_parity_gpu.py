@@ -260,6 +260,56 @@ def test_balanced_split_matches_plain_launch(ocn, oracle, torch_gpu, N, C, H, K)
     np.testing.assert_allclose(y1, y0, rtol=0, atol=2e-6 * np.abs(y0).max())
 
 
+# ---------------------------------------------------------------- layout shims
+
+@pytest.mark.parametrize("N,C,H,W,K", [(32, 8, 8, 8, 64), (64, 64, 56, 56, 64), (96, 1030, 5, 3, 33), (1, 1, 1, 1, 1)])
+def test_layout_shims_are_exact_permutations(ocn, torch_gpu, N, C, H, W, K):
+    # the reference's data_cpy transposes (src/openCNN_winograd.cu:147-153,230,235): bit-exact,
+    # checked against numpy; C = 1030 is beyond data_cpy's C <= 1024 launch limit
+    print(f"shims N={N} C={C} H={H} W={W} K={K}", flush=True)
+    torch = torch_gpu
+    nchw = ocn.synth_input(N, C, H, W, seed=5, layout=ocn.INPUT_NCHW)
+    src = torch.from_numpy(nchw).cuda()
+    dst = torch.full((C, H, W, N), float("nan"), device="cuda")
+    ocn.nchw_to_chwn(src, dst, N, C, H, W)
+    torch.cuda.synchronize()
+    assert np.array_equal(dst.cpu().numpy(), nchw.transpose(1, 2, 3, 0))
+    assert np.array_equal(dst.cpu().numpy(), ocn.synth_input(N, C, H, W, seed=5))
+    back = torch.full((N, C, H, W), float("nan"), device="cuda")
+    ocn.khwn_to_nkhw(dst, back, N, C, H, W)  # a CHWN tensor is a KHWN tensor with K = C
+    torch.cuda.synchronize()
+    assert np.array_equal(back.cpu().numpy(), nchw)
+    kc = min(C, 64)
+    kcrs = ocn.synth_filter(K, kc, seed=6, layout=ocn.FILTER_KCRS)
+    fsrc = torch.from_numpy(kcrs).cuda()
+    fdst = torch.full((kc, 3, 3, K), float("nan"), device="cuda")
+    ocn.kcrs_to_crsk(fsrc, fdst, K, kc)
+    torch.cuda.synchronize()
+    assert np.array_equal(fdst.cpu().numpy(), ocn.synth_filter(K, kc, seed=6))
+
+
+def test_nchw_pipeline_end_to_end(ocn, oracle, torch_gpu):
+    # the reference bench's data flow: NCHW / KCRS tensors -> shims -> convolutionForward -> NCHW
+    print("nchw pipeline", flush=True)
+    torch = torch_gpu
+    N, C, H, K = 64, 32, 12, 64
+    nchw = ocn.synth_input(N, C, H, H, seed=SEED_X, layout=ocn.INPUT_NCHW)
+    kcrs = ocn.synth_filter(K, C, seed=SEED_W, layout=ocn.FILTER_KCRS)
+    xs, ws_ = torch.from_numpy(nchw).cuda(), torch.from_numpy(kcrs).cuda()
+    xd, wd = torch.empty(C * H * H * N, device="cuda"), torch.empty(C * 9 * K, device="cuda")
+    yd, yn = torch.empty(K * H * H * N, device="cuda"), torch.empty((N, K, H, H), device="cuda")
+    wsp = torch.empty(C * 16 * K, device="cuda")
+    ocn.nchw_to_chwn(xs, xd, N, C, H, H)
+    ocn.kcrs_to_crsk(ws_, wd, K, C)
+    td = ocn.tiles_dim(H)
+    ocn.convolutionForward(xd, H, H, wd, H, H, N, K, yd, wsp, K * N * H * H, td, N, 4, td * 4, C, K, C, 3, 3, 4, 2)
+    ocn.khwn_to_nkhw(yd, yn, N, K, H, H)
+    torch.cuda.synchronize()
+    want = oracle.direct_conv_f64(nchw.transpose(1, 2, 3, 0), kcrs.transpose(1, 2, 3, 0)).transpose(3, 0, 1, 2)
+    rel, _, _ = oracle.compare(yn.cpu().numpy(), np.ascontiguousarray(want))
+    assert rel <= 1e-5
+
+
 # ---------------------------------------------------------------- fp16 / bf16 GEMM operands
 
 # bounds against the fp64 direct convolution: unit round-offs 2^-11 (fp16) and 2^-8 (bf16) on
