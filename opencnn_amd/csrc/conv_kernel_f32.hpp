@@ -415,7 +415,10 @@ __global__ void __launch_bounds__(256) wino_f32_fused_lds(ConvArgs a) {
         __builtin_amdgcn_sched_barrier(0);
         if (s == 0) load_u(a, w, lane, u[1], 2 * i + 1);
         if (s == 2) load_u(a, w, lane, u[0], 2 * i + 2);
-        if (s == 1) load_patches(i + 2);
+        // patches of chunk i+2: 16 loads per owned step; with two owned steps (KW = 2) the second
+        // batch goes behind the MFMAs of step 3, which has no other loads
+        if (s == 1) load_patch(a, w, d[0], (i + 2) * 4 + kw * SPW);
+        if (s == 3 && SPW == 2) load_patch(a, w, d[1], (i + 2) * 4 + kw * SPW + 1);
         if (s < 3) read_v(v[(s + 1) & 1], buf, s + 1);
 #pragma unroll
         for (int p = 0; p < 16; ++p)
@@ -426,7 +429,7 @@ __global__ void __launch_bounds__(256) wino_f32_fused_lds(ConvArgs a) {
 #pragma unroll
         for (int p = 0; p < 16; ++p) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // one MFMA
-          if (s != 3) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
+          if (s != 3 || SPW == 2) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
           if (s != 3 && (p & 1)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
         }
         __builtin_amdgcn_sched_barrier(0);
