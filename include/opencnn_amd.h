@@ -111,7 +111,9 @@ int opencnn_set_stream(void *stream);
  * Which fused kernel later calls launch.  The reference picks its variant at compile time
  * (-DBASE / -DOPTSTS64 / -DOPTSTS64_CMP / -DOPTLDS64, Makefile:3,8); here it is a run-time
  * switch so both can be measured in one process.
- *   OPENCNN_KERNEL_AUTO      the LDS variant when filt_k % 64 == 0, else the register variant
+ *   OPENCNN_KERNEL_AUTO      the LDS variant when filt_k % 64 == 0 (as one continuous pipeline
+ *                            over all tiles of a workgroup when the balanced split is in use),
+ *                            else the register variant
  *   OPENCNN_KERNEL_REGISTER  every wave transforms its own input patches; no LDS, no barriers
  *   OPENCNN_KERNEL_LDS       the waves of a workgroup that share a column tile split the input
  *                            transform and exchange it through LDS (needs filt_k % 64 == 0,

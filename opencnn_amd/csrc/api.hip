@@ -189,15 +189,27 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   int cus = 0;
   if (int e = compute_units(&cus)) return e;
   const bool balanced = g_balance.load() != 0 && a.nblocks > cus && a.nblocks % cus != 0 &&
-                        cus % 8 == 0 && cus <= opencnn::kMaxBalancedBlocks;
+                        cus % 8 == 0 && cus <= opencnn::kMaxBalancedBlocks &&
+                        (long long)a.nblocks * (in_c / 8) <= kMaxElems;
   if (balanced) grid = dim3(cus);
+  // The continuous pipeline pays off when a workgroup walks several tiles; for a single tile
+  // per workgroup the plain LDS kernel has less scalar work per load.
+  const bool stream = balanced && g_variant.load() != OPENCNN_KERNEL_LDS;
   if (kw == 4) {
-    if (balanced)
+    if (stream && balanced)
+      opencnn::wino_f32_stream<4, true><<<grid, block, lds_bytes, st>>>(a);
+    else if (stream)
+      opencnn::wino_f32_stream<4, false><<<grid, block, lds_bytes, st>>>(a);
+    else if (balanced)
       opencnn::wino_f32_fused_lds<4, true><<<grid, block, lds_bytes, st>>>(a);
     else
       opencnn::wino_f32_fused_lds<4, false><<<grid, block, lds_bytes, st>>>(a);
   } else {
-    if (balanced)
+    if (stream && balanced)
+      opencnn::wino_f32_stream<2, true><<<grid, block, lds_bytes, st>>>(a);
+    else if (stream)
+      opencnn::wino_f32_stream<2, false><<<grid, block, lds_bytes, st>>>(a);
+    else if (balanced)
       opencnn::wino_f32_fused_lds<2, true><<<grid, block, lds_bytes, st>>>(a);
     else
       opencnn::wino_f32_fused_lds<2, false><<<grid, block, lds_bytes, st>>>(a);

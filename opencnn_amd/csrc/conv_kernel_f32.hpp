@@ -472,4 +472,245 @@ __global__ void __launch_bounds__(256) wino_f32_fused_lds(ConvArgs a) {
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// Kernel C: kernel B as ONE continuous software pipeline over the workgroup's whole range of
+// (tile, chunk) units.  In kernel B every tile (or part of a tile) starts with a prologue whose
+// first loads nobody prefetched (about 2 us of idle matrix pipe per tile, 8-10 % of a tile of
+// 8-16 chunks).  Here the loads run two units ahead of the MFMAs ACROSS tile boundaries: while
+// the last chunk of a tile is being multiplied, the first chunks of the next tile are already
+// being loaded, transformed and published, so a tile boundary costs the output transform and
+// the zeroing of the accumulators, nothing else.
+//
+// To make tile switches cheap the per-tile state is scalar: the 16 patch offsets of kernels A
+// and B (16 VGPRs per lane) become one per-lane base offset plus 16 wave-uniform scalar offsets,
+// and the zero padding is a per-element choice between the real buffer descriptor and an empty
+// one (a load through an empty descriptor returns 0 without touching memory).
+struct TileState {
+  int kg, ng, ty, tx;  // wave-uniform
+  int live;            // 0: this wave's column tile does not exist (stores dropped)
+  unsigned vmask;      // bit i*4+j: patch element (i,j) lies inside the image
+  int vbase;           // per lane: byte offset of (channel hsel, row 2ty, col 2tx, n) in a slab
+};
+
+template <int KW>
+__device__ __forceinline__ void decode_state(const ConvArgs& a, int T, int kw, int cw, int lane, TileState& t) {
+  constexpr int CW = 4 / KW;
+  const int kblocks = a.kgroups / KW;
+  const int cg_raw = (T / kblocks) * CW + cw;
+  t.live = cg_raw < a.colgroups;
+  const int cg = t.live ? cg_raw : a.colgroups - 1;
+  const int tile = cg / a.ngroups;
+  t.kg = (T % kblocks) * KW + kw;
+  t.ng = cg - tile * a.ngroups;
+  t.ty = tile / a.tiles_w;
+  t.tx = tile - t.ty * a.tiles_w;
+  unsigned m = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int hh = 2 * t.ty - 1 + i, ww = 2 * t.tx - 1 + j;
+      if (hh >= 0 && hh < a.H && ww >= 0 && ww < a.W) m |= 1u << (i * 4 + j);
+    }
+  t.vmask = m;
+  t.vbase = (((lane >> 5) * a.H * a.W + 2 * t.ty * a.W + 2 * t.tx) * a.N + t.ng * 32 + (lane & 31)) * 4;
+}
+
+// Patch of MFMA step `step` (channels 2*step + hsel) of the tile in `t`.
+__device__ __forceinline__ void load_patch_s(const ConvArgs& a, const TileState& t, float (&d)[16], int step) {
+  const size_t HWN = (size_t)a.H * a.W * a.N;
+  const int st = __builtin_amdgcn_readfirstlane(step);
+  const int rowb = a.W * a.N * 4, colb = a.N * 4;
+  // The base is moved back by one row and one column so that the per-lane offset is never
+  // negative (it is range-checked on its own); valid elements still address inside x.
+  const char* base = reinterpret_cast<const char*>(a.x + (size_t)st * 2 * HWN) - rowb - colb;
+  const unsigned span = (unsigned)(2 * HWN * sizeof(float)) + 4u * (unsigned)rowb;
+  const __amdgpu_buffer_rsrc_t real = make_rsrc(base, span);
+  const __amdgpu_buffer_rsrc_t none = make_rsrc(base, 0u);
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const bool ok = (t.vmask >> (i * 4 + j)) & 1u;
+      d[i * 4 + j] = __builtin_bit_cast(
+          float, __builtin_amdgcn_raw_buffer_load_b32(ok ? real : none, t.vbase, i * rowb + j * colb, 0));
+    }
+}
+
+__device__ __forceinline__ void load_u_s(const ConvArgs& a, int kg, int lane, v2f (&u)[16], int quad) {
+  const int Q = a.C >> 2;
+  const __amdgpu_buffer_rsrc_t ru = make_rsrc(a.usw, (unsigned)((size_t)a.C * 16 * a.K * sizeof(float)));
+  const int soff = __builtin_amdgcn_readfirstlane((kg * Q + quad) * (16 * 64 * 8));
+#pragma unroll
+  for (int p = 0; p < 16; ++p)
+    u[p] = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(ru, lane * 8 + p * 512, soff, 0));
+}
+
+template <int KW, bool BALANCED>
+__global__ void __launch_bounds__(256) wino_f32_stream(ConvArgs a) {
+  constexpr int SPW = 4 / KW;
+  extern __shared__ float lds[];  // [CW][2][4][16][64]
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int kw = wave % KW, cw = wave / KW;
+  const int L = logical_block();
+  const int chunks = a.C >> 3;
+
+  // units [begin, begin + n) of this workgroup; unit = tile * chunks + chunk
+  int begin, n;
+  if (BALANCED) {
+    const long long total = (long long)a.nblocks * chunks;
+    begin = (int)(total * L / gridDim.x);
+    n = (int)(total * (L + 1) / gridDim.x) - begin;
+  } else {
+    if (L >= a.nblocks) return;  // whole workgroup
+    begin = L * chunks;
+    n = chunks;
+  }
+  const int T_first = begin / chunks, c_first = begin - T_first * chunks;
+
+  float* vl = lds + cw * (2 * 4 * 16 * 64) + lane;
+  auto vaddr = [&](int buf, int step, int p) { return vl + ((buf * 4 + step) * 16 + p) * 64; };
+  auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+  v2f u[2][16];      // filter operands of the current / next quad
+  float d[SPW][16];  // this wave's share of the patches of the unit after next, in flight
+  float v[2][16];    // B operands of the current / next step
+
+  auto transform_to_lds = [&](int buf) {
+#pragma unroll
+    for (int j = 0; j < SPW; ++j) {
+      float t[16];
+      input_transform(d[j], t);
+#pragma unroll
+      for (int p = 0; p < 16; ++p) *vaddr(buf, kw * SPW + j, p) = t[p];
+    }
+  };
+  auto read_v = [&](float (&dst)[16], int buf, int step) {
+#pragma unroll
+    for (int p = 0; p < 16; ++p) dst[p] = *vaddr(buf, step, p);
+  };
+
+  // Cursors.  M: the unit being multiplied.  P: the unit whose patches are loaded (M + 2).
+  // Q: the unit whose first filter quad is loaded (M + 1).  Past the last unit they stay on it
+  // (the loads are repeated and never used).
+  TileState tm, tp;
+  int Tp = T_first, cp = c_first;  // P
+  int Tq = T_first, cq = c_first;  // Q
+  int kgq;
+  decode_state<KW>(a, T_first, kw, cw, lane, tp);
+  tm = tp;
+  kgq = tp.kg;
+  auto advance_p = [&](int unit_index) {  // move P to begin + unit_index (if it exists)
+    if (unit_index < n) {
+      if (++cp == chunks) {
+        cp = 0;
+        ++Tp;
+        decode_state<KW>(a, Tp, kw, cw, lane, tp);
+      }
+    }
+  };
+  auto advance_q = [&](int unit_index) {
+    if (unit_index < n) {
+      if (++cq == chunks) {
+        cq = 0;
+        ++Tq;
+        kgq = ((Tq % (a.kgroups / KW)) * KW) + kw;
+      }
+    }
+  };
+  auto load_patches = [&](int j) { load_patch_s(a, tp, d[j], cp * 4 + kw * SPW + j); };
+
+  // prologue (once per workgroup): unit 0 -> buf 0; unit 1 patches in flight; first quad in u[0]
+  load_u_s(a, kgq, lane, u[0], 2 * cq);
+#pragma unroll
+  for (int j = 0; j < SPW; ++j) load_patches(j);
+  transform_to_lds(0);
+  advance_p(1);
+#pragma unroll
+  for (int j = 0; j < SPW; ++j) load_patches(j);
+  lds_barrier();
+  read_v(v[0], 0, 0);
+
+  int Tm = T_first, cm = c_first, g = 0;
+  for (;;) {
+    // one tile, or the part of it that falls into this workgroup's range: chunks cm .. seg_end-1
+    const int seg_first = cm;
+    const int seg_end = (n - g) < (chunks - cm) ? cm + (n - g) : chunks;
+    v16f acc[16];
+#pragma unroll
+    for (int p = 0; p < 16; ++p)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[p][r] = 0.0f;
+
+    for (; cm < seg_end; ++cm, ++g) {
+      const int buf = g & 1;
+      advance_p(g + 2);
+      advance_q(g + 1);
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (s == 0) transform_to_lds(buf ^ 1);  // unit g+1: one VALU burst, then its LDS writes
+        __builtin_amdgcn_sched_barrier(0);
+        if (s == 0) load_u_s(a, tm.kg, lane, u[1], 2 * cm + 1);
+        if (s == 2) load_u_s(a, kgq, lane, u[0], 2 * cq);
+        if (s == 1) load_patches(0);
+        if (s == 3 && SPW == 2) load_patches(1);
+        if (s < 3) read_v(v[(s + 1) & 1], buf, s + 1);
+#pragma unroll
+        for (int p = 0; p < 16; ++p)
+          acc[p] = __builtin_amdgcn_mfma_f32_32x32x2f32(u[s >> 1][p][s & 1], v[s & 1][p], acc[p], 0, 0, 0);
+#pragma unroll
+        for (int p = 0; p < 16; ++p) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+          if (s != 3 || SPW == 2) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
+          if (s != 3 && (p & 1)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      lds_barrier();
+      read_v(v[0], buf ^ 1, 0);
+    }
+
+    // output transform of the finished (part of the) tile: store, or merge with the other part
+    WaveTile w;  // position only; store_tile does not use the patch offsets
+    w.kg = tm.kg;
+    w.ng = tm.ng;
+    w.ty = tm.ty;
+    w.tx = tm.tx;
+    w.hsel = lane >> 5;
+    w.nl = lane & 31;
+    if (tm.live) {
+      if (!BALANCED || (seg_first == 0 && seg_end == chunks)) {
+        store_tile<kStorePlain>(a, w, acc);
+      } else {
+        unsigned* sync = g_split_sync + ((seg_first > 0 ? L - 1 : L) * 4 + wave) * 2;
+        unsigned ticket = 0;
+        if (lane == 0) ticket = __hip_atomic_fetch_add(sync, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        ticket = __builtin_amdgcn_readfirstlane(ticket);
+        if (ticket == 0) {
+          store_tile<kStorePublish>(a, w, acc);
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          if (lane == 0) __hip_atomic_store(sync + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        } else {
+          for (int spin = 0; spin < (1 << 22); ++spin) {
+            if (__hip_atomic_load(sync + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0) break;
+            __builtin_amdgcn_s_sleep(8);
+          }
+          asm volatile("" ::: "memory");
+          store_tile<kStoreMerge>(a, w, acc);
+          if (lane == 0) {
+            __hip_atomic_store(sync, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            __hip_atomic_store(sync + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+          }
+        }
+      }
+    }
+    if (g >= n) break;
+    ++Tm;
+    cm = 0;
+    decode_state<KW>(a, Tm, kw, cw, lane, tm);
+  }
+}
+
 }  // namespace opencnn
