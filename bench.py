@@ -22,6 +22,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
+PEAK_F16_MFMA_TFLOPS = 2500.0  # dense fp16 / bf16 matrix peak
 PEAK_HBM_GBS = 8000.0
 
 # name -> (N, C, H=W, K, input range, filter distribution)
@@ -31,7 +32,10 @@ LAYERS = {
     "resnet_n128_c128_h28_k128": (128, 128, 28, 128, (-1.0, 1.0), "he"),
     "deep_n128_c256_h14_k256": (128, 256, 14, 256, (0.0, 1.0), "he"),
     "deep_n128_c512_h7_k512": (128, 512, 7, 512, (0.0, 1.0), "he"),
+    # reduced-precision configuration: fp16 / bf16 GEMM operands, fp32 transforms and accumulation
+    "reduced_n128_c256_h14_k256": (128, 256, 14, 256, (-1.0, 1.0), "he"),
 }
+FP32_LAYERS = [k for k in LAYERS if not k.startswith("reduced")]
 DEFAULT_WORKLOAD = "resnet_n64_c64_h56_k64"
 
 # HBM bytes per launch of the fused kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
@@ -108,9 +112,9 @@ def cpu_baseline(layer):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(LAYERS))
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(FP32_LAYERS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-layers", action="store_true", help="skip the per-layer table")
     args = ap.parse_args()
@@ -163,7 +167,7 @@ def main():
                    "W": layer.H, "K": layer.K, "pad": 1, "stride": 1,
                    "layout": "CHWN in, CRSK filters, KHWN out"},
         "roofline": {
-            "kernel": "wino_f32_fused",
+            "kernel": "wino_f32_stream / wino_f32_fused_lds (fused Winograd kernel)",
             "bound": "mfma",
             "achieved": achieved,
             "peak": PEAK_FP32_MFMA_TFLOPS,
@@ -192,15 +196,24 @@ def main():
         rows = []
         for name in LAYERS:
             lay = layer if name == layer.name else Layer(ocn, torch, name)
-            tot, mn, fx = lay.kernel_times(3, 50)
             d, m, b = work(lay.N, lay.C, lay.H, lay.K)
-            rows.append({
-                "workload": name, "ms_per_layer": tot, "ms_fused_kernel": mn, "ms_filter_transform": fx,
-                "effective_tflops": d / (tot * 1e-3) / 1e12,
-                "mfma_tflops": m / (mn * 1e-3) / 1e12,
-                "mfma_frac_of_peak": m / (mn * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS,
-                "hbm_gbs_at_min_bytes": b / (tot * 1e-3) / 1e9,
-            })
+            precisions = [("f32", ocn.F32, PEAK_FP32_MFMA_TFLOPS)]
+            if name.startswith("reduced"):
+                precisions = [("f16", ocn.F16, PEAK_F16_MFMA_TFLOPS), ("bf16", ocn.BF16, PEAK_F16_MFMA_TFLOPS)]
+            for label, prec, peak in precisions:
+                try:
+                    ocn.set_operand_precision(prec)
+                    tot, mn, fx = lay.kernel_times(20, 200)
+                finally:
+                    ocn.set_operand_precision(ocn.F32)
+                rows.append({
+                    "workload": name, "gemm_operands": label, "ms_per_layer": tot, "ms_fused_kernel": mn,
+                    "ms_filter_transform": fx,
+                    "effective_tflops": d / (tot * 1e-3) / 1e12,
+                    "mfma_tflops": m / (mn * 1e-3) / 1e12,
+                    "mfma_frac_of_peak": m / (mn * 1e-3) / 1e12 / peak,
+                    "hbm_gbs_at_min_bytes": b / (tot * 1e-3) / 1e9,
+                })
             del lay
         out["layers"] = rows
 
