@@ -197,18 +197,18 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   const bool stream = balanced && g_variant.load() != OPENCNN_KERNEL_LDS;
   if (kw == 4) {
     if (stream && balanced)
-      opencnn::wino_f32_stream<4, true><<<grid, block, lds_bytes, st>>>(a);
+      opencnn::wino_f32_stream<4, true, true><<<grid, block, lds_bytes, st>>>(a);
     else if (stream)
-      opencnn::wino_f32_stream<4, false><<<grid, block, lds_bytes, st>>>(a);
+      opencnn::wino_f32_stream<4, false, true><<<grid, block, lds_bytes, st>>>(a);
     else if (balanced)
       opencnn::wino_f32_fused_lds<4, true><<<grid, block, lds_bytes, st>>>(a);
     else
       opencnn::wino_f32_fused_lds<4, false><<<grid, block, lds_bytes, st>>>(a);
   } else {
     if (stream && balanced)
-      opencnn::wino_f32_stream<2, true><<<grid, block, lds_bytes, st>>>(a);
+      opencnn::wino_f32_stream<2, true, false><<<grid, block, lds_bytes, st>>>(a);
     else if (stream)
-      opencnn::wino_f32_stream<2, false><<<grid, block, lds_bytes, st>>>(a);
+      opencnn::wino_f32_stream<2, false, false><<<grid, block, lds_bytes, st>>>(a);
     else if (balanced)
       opencnn::wino_f32_fused_lds<2, true><<<grid, block, lds_bytes, st>>>(a);
     else

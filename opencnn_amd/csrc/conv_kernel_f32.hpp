@@ -481,29 +481,46 @@ __global__ void __launch_bounds__(256) wino_f32_fused_lds(ConvArgs a) {
 // being loaded, transformed and published, so a tile boundary costs the output transform and
 // the zeroing of the accumulators, nothing else.
 //
-// To make tile switches cheap the per-tile state is scalar: the 16 patch offsets of kernels A
-// and B (16 VGPRs per lane) become one per-lane base offset plus 16 wave-uniform scalar offsets,
-// and the zero padding is a per-element choice between the real buffer descriptor and an empty
-// one (a load through an empty descriptor returns 0 without touching memory).
+// Three cursors walk the unit range: P (patch loads, two units ahead of the MFMAs), Q (first
+// filter quad, one unit ahead) and M (the MFMAs and the epilogue).  Q and M only need
+// wave-uniform tile coordinates.  P addresses its 16 patch elements in one of two ways:
+//   SCALAR_PATCH = false  16 per-lane byte offsets (WaveTile::voff), re-decoded on a tile switch;
+//   SCALAR_PATCH = true   one per-lane base offset plus 16 wave-uniform scalar offsets, the zero
+//                         padding being a per-element choice between the real buffer descriptor
+//                         and an empty one (a load through it returns 0 without touching memory).
+// Which one hipcc turns into the faster loop depends on the register pressure of the
+// instantiation (measured: scalar for KW = 4, per-lane for KW = 2).
 struct TileState {
   int kg, ng, ty, tx;  // wave-uniform
   int live;            // 0: this wave's column tile does not exist (stores dropped)
-  unsigned vmask;      // bit i*4+j: patch element (i,j) lies inside the image
-  int vbase;           // per lane: byte offset of (channel hsel, row 2ty, col 2tx, n) in a slab
 };
 
 template <int KW>
-__device__ __forceinline__ void decode_state(const ConvArgs& a, int T, int kw, int cw, int lane, TileState& t) {
+__device__ __forceinline__ int column_tile_of(const ConvArgs& a, int T, int cw, int& live) {
   constexpr int CW = 4 / KW;
-  const int kblocks = a.kgroups / KW;
-  const int cg_raw = (T / kblocks) * CW + cw;
-  t.live = cg_raw < a.colgroups;
-  const int cg = t.live ? cg_raw : a.colgroups - 1;
+  const int cg_raw = (T / (a.kgroups / KW)) * CW + cw;
+  live = cg_raw < a.colgroups;
+  // A workgroup whose last column tile does not exist keeps those waves busy on a copy of
+  // the last real one (they must take part in the barriers) and drops their stores.
+  return live ? cg_raw : a.colgroups - 1;
+}
+
+template <int KW>
+__device__ __forceinline__ void decode_state(const ConvArgs& a, int T, int kw, int cw, TileState& t) {
+  const int cg = column_tile_of<KW>(a, T, cw, t.live);
   const int tile = cg / a.ngroups;
-  t.kg = (T % kblocks) * KW + kw;
+  t.kg = (T % (a.kgroups / KW)) * KW + kw;
   t.ng = cg - tile * a.ngroups;
   t.ty = tile / a.tiles_w;
   t.tx = tile - t.ty * a.tiles_w;
+}
+
+struct ScalarPatch {
+  unsigned vmask;  // bit i*4+j: patch element (i,j) lies inside the image (wave-uniform)
+  int vbase;       // per lane: byte offset of (channel hsel, row 2ty, col 2tx, n) in a slab
+};
+
+__device__ __forceinline__ void decode_scalar_patch(const ConvArgs& a, const TileState& t, int lane, ScalarPatch& sp) {
   unsigned m = 0;
 #pragma unroll
   for (int i = 0; i < 4; ++i)
@@ -512,12 +529,12 @@ __device__ __forceinline__ void decode_state(const ConvArgs& a, int T, int kw, i
       const int hh = 2 * t.ty - 1 + i, ww = 2 * t.tx - 1 + j;
       if (hh >= 0 && hh < a.H && ww >= 0 && ww < a.W) m |= 1u << (i * 4 + j);
     }
-  t.vmask = m;
-  t.vbase = (((lane >> 5) * a.H * a.W + 2 * t.ty * a.W + 2 * t.tx) * a.N + t.ng * 32 + (lane & 31)) * 4;
+  sp.vmask = m;
+  sp.vbase = (((lane >> 5) * a.H * a.W + 2 * t.ty * a.W + 2 * t.tx) * a.N + t.ng * 32 + (lane & 31)) * 4;
 }
 
-// Patch of MFMA step `step` (channels 2*step + hsel) of the tile in `t`.
-__device__ __forceinline__ void load_patch_s(const ConvArgs& a, const TileState& t, float (&d)[16], int step) {
+// Patch of MFMA step `step` (channels 2*step + hsel) through scalar offsets.
+__device__ __forceinline__ void load_patch_s(const ConvArgs& a, const ScalarPatch& sp, float (&d)[16], int step) {
   const size_t HWN = (size_t)a.H * a.W * a.N;
   const int st = __builtin_amdgcn_readfirstlane(step);
   const int rowb = a.W * a.N * 4, colb = a.N * 4;
@@ -531,9 +548,9 @@ __device__ __forceinline__ void load_patch_s(const ConvArgs& a, const TileState&
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const bool ok = (t.vmask >> (i * 4 + j)) & 1u;
+      const bool ok = (sp.vmask >> (i * 4 + j)) & 1u;
       d[i * 4 + j] = __builtin_bit_cast(
-          float, __builtin_amdgcn_raw_buffer_load_b32(ok ? real : none, t.vbase, i * rowb + j * colb, 0));
+          float, __builtin_amdgcn_raw_buffer_load_b32(ok ? real : none, sp.vbase, i * rowb + j * colb, 0));
     }
 }
 
@@ -546,7 +563,7 @@ __device__ __forceinline__ void load_u_s(const ConvArgs& a, int kg, int lane, v2
     u[p] = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(ru, lane * 8 + p * 512, soff, 0));
 }
 
-template <int KW, bool BALANCED>
+template <int KW, bool BALANCED, bool SCALAR_PATCH>
 __global__ void __launch_bounds__(256) wino_f32_stream(ConvArgs a) {
   constexpr int SPW = 4 / KW;
   extern __shared__ float lds[];  // [CW][2][4][16][64]
@@ -594,19 +611,32 @@ __global__ void __launch_bounds__(256) wino_f32_stream(ConvArgs a) {
   // Cursors.  M: the unit being multiplied.  P: the unit whose patches are loaded (M + 2).
   // Q: the unit whose first filter quad is loaded (M + 1).  Past the last unit they stay on it
   // (the loads are repeated and never used).
-  TileState tm, tp;
+  TileState tm;
+  WaveTile wp;     // used when !SCALAR_PATCH
+  ScalarPatch sp;  // used when SCALAR_PATCH
   int Tp = T_first, cp = c_first;  // P
   int Tq = T_first, cq = c_first;  // Q
   int kgq;
-  decode_state<KW>(a, T_first, kw, cw, lane, tp);
-  tm = tp;
-  kgq = tp.kg;
+  auto decode_p = [&]() {
+    if (SCALAR_PATCH) {
+      TileState t;
+      decode_state<KW>(a, Tp, kw, cw, t);
+      decode_scalar_patch(a, t, lane, sp);
+    } else {
+      int live;
+      const int cg = column_tile_of<KW>(a, Tp, cw, live);
+      decode_tile(a, (Tp % (a.kgroups / KW)) * KW + kw, cg, lane, wp);
+    }
+  };
+  decode_p();
+  decode_state<KW>(a, T_first, kw, cw, tm);
+  kgq = tm.kg;
   auto advance_p = [&](int unit_index) {  // move P to begin + unit_index (if it exists)
     if (unit_index < n) {
       if (++cp == chunks) {
         cp = 0;
         ++Tp;
-        decode_state<KW>(a, Tp, kw, cw, lane, tp);
+        decode_p();
       }
     }
   };
@@ -619,7 +649,12 @@ __global__ void __launch_bounds__(256) wino_f32_stream(ConvArgs a) {
       }
     }
   };
-  auto load_patches = [&](int j) { load_patch_s(a, tp, d[j], cp * 4 + kw * SPW + j); };
+  auto load_patches = [&](int j) {
+    if (SCALAR_PATCH)
+      load_patch_s(a, sp, d[j], cp * 4 + kw * SPW + j);
+    else
+      load_patch(a, wp, d[j], cp * 4 + kw * SPW + j);
+  };
 
   // prologue (once per workgroup): unit 0 -> buf 0; unit 1 patches in flight; first quad in u[0]
   load_u_s(a, kgq, lane, u[0], 2 * cq);
@@ -684,32 +719,32 @@ __global__ void __launch_bounds__(256) wino_f32_stream(ConvArgs a) {
       if (!BALANCED || (seg_first == 0 && seg_end == chunks)) {
         store_tile<kStorePlain>(a, w, acc);
       } else {
-        unsigned* sync = g_split_sync + ((seg_first > 0 ? L - 1 : L) * 4 + wave) * 2;
-        unsigned ticket = 0;
-        if (lane == 0) ticket = __hip_atomic_fetch_add(sync, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-        ticket = __builtin_amdgcn_readfirstlane(ticket);
-        if (ticket == 0) {
+        // The roles are fixed by position, no ticket needed: a segment that starts inside a
+        // tile (seg_first > 0) is this workgroup's FIRST one, finishes early and publishes; the
+        // other part of that tile is the LAST segment of the previous workgroup, finishes late
+        // and merges.  (Ranges are at least one tile long, so a segment is never both.)
+        if (seg_first > 0) {
+          unsigned* flag = g_split_sync + ((L - 1) * 4 + wave) * 2 + 1;
           store_tile<kStorePublish>(a, w, acc);
-          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-          if (lane == 0) __hip_atomic_store(sync + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // write-through stores acknowledged
+          if (lane == 0) __hip_atomic_store(flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         } else {
+          unsigned* flag = g_split_sync + (L * 4 + wave) * 2 + 1;
+          // normally set long ago; bounded wait all the same (never hang the GPU on a bug)
           for (int spin = 0; spin < (1 << 22); ++spin) {
-            if (__hip_atomic_load(sync + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0) break;
+            if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0) break;
             __builtin_amdgcn_s_sleep(8);
           }
-          asm volatile("" ::: "memory");
+          asm volatile("" ::: "memory");  // the partial result is read after the flag, not before
           store_tile<kStoreMerge>(a, w, acc);
-          if (lane == 0) {
-            __hip_atomic_store(sync, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-            __hip_atomic_store(sync + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-          }
+          if (lane == 0) __hip_atomic_store(flag, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         }
       }
     }
     if (g >= n) break;
     ++Tm;
     cm = 0;
-    decode_state<KW>(a, Tm, kw, cw, lane, tm);
+    decode_state<KW>(a, Tm, kw, cw, tm);
   }
 }
 
