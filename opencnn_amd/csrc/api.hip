@@ -146,6 +146,7 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
     const long long hblocks = (long long)((a.colgroups + hcw - 1) / hcw) * (a.kgroups / hkw);
     REQUIRE(hblocks <= kMaxElems / 8);
     a.nblocks = (int)hblocks;
+    a.colblocks = (a.colgroups + hcw - 1) / hcw;
     dim3 hgrid(((a.nblocks + 7) / 8) * 8), hblock(256);
     const size_t hlds = (size_t)hcw * 3 * 16 * 2 * 4 * 32 * sizeof(unsigned);
     const bool bf = precision == OPENCNN_BF16;
@@ -177,6 +178,7 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   const long long nblocks = colblocks * (a.kgroups / kw);
   REQUIRE(nblocks <= kMaxElems / 8);
   a.nblocks = (int)nblocks;
+  a.colblocks = (int)colblocks;
   const int per_xcd = (a.nblocks + 7) / 8;
   dim3 grid(per_xcd * 8), block(256);
   const size_t lds_bytes = (size_t)cw * 2 * 4 * 16 * 64 * sizeof(float);

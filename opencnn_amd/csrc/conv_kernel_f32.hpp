@@ -44,7 +44,11 @@ struct ConvArgs {
   int ngroups;           // N / 32
   int colgroups;         // tiles_h * tiles_w * ngroups   (wave-level column tiles)
   int kgroups;           // K / 32
-  int nblocks;           // workgroup tiles: column blocks x filter blocks
+  int nblocks;           // workgroup tiles: filter blocks x column blocks
+  int colblocks;         // column blocks; workgroup tile T = filter block T / colblocks,
+                         // column block T % colblocks (LDS kernels): an XCD's contiguous
+                         // range of tiles then needs one filter block's share of Ww, which
+                         // fits its L2, instead of all of it
 };
 
 // V = B^T d B, columns first then rows (src/convolutionForward_32x64x8.cu:59-80).
@@ -334,7 +338,6 @@ __global__ void __launch_bounds__(256) wino_f32_fused_lds(ConvArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int kw = wave % KW, cw = wave / KW;
   const int L = logical_block();
-  const int kblocks = a.kgroups / KW;
   const int chunks = a.C >> 3;
 
   // chunk-units [unit, end) of this workgroup; unit = tile * chunks + chunk
@@ -361,13 +364,13 @@ __global__ void __launch_bounds__(256) wino_f32_fused_lds(ConvArgs a) {
     const int c1 = (end - unit) < (long long)(chunks - c0) ? c0 + (int)(end - unit) : chunks;
     unit += c1 - c0;
 
-    const int cg_raw = (T / kblocks) * CW + cw;
+    const int cg_raw = (T % a.colblocks) * CW + cw;
     const bool live = cg_raw < a.colgroups;
     // A workgroup whose last column tile does not exist keeps those waves busy on a copy of
     // the last real one (they must take part in the barriers) and drops their stores.
     const int cg = live ? cg_raw : a.colgroups - 1;
     WaveTile w;
-    decode_tile(a, (T % kblocks) * KW + kw, cg, lane, w);
+    decode_tile(a, (T / a.colblocks) * KW + kw, cg, lane, w);
 
     v16f acc[16];
 #pragma unroll
@@ -498,7 +501,7 @@ struct TileState {
 template <int KW>
 __device__ __forceinline__ int column_tile_of(const ConvArgs& a, int T, int cw, int& live) {
   constexpr int CW = 4 / KW;
-  const int cg_raw = (T / (a.kgroups / KW)) * CW + cw;
+  const int cg_raw = (T % a.colblocks) * CW + cw;
   live = cg_raw < a.colgroups;
   // A workgroup whose last column tile does not exist keeps those waves busy on a copy of
   // the last real one (they must take part in the barriers) and drops their stores.
@@ -509,7 +512,7 @@ template <int KW>
 __device__ __forceinline__ void decode_state(const ConvArgs& a, int T, int kw, int cw, TileState& t) {
   const int cg = column_tile_of<KW>(a, T, cw, t.live);
   const int tile = cg / a.ngroups;
-  t.kg = (T % (a.kgroups / KW)) * KW + kw;
+  t.kg = (T / a.colblocks) * KW + kw;
   t.ng = cg - tile * a.ngroups;
   t.ty = tile / a.tiles_w;
   t.tx = tile - t.ty * a.tiles_w;
@@ -625,7 +628,7 @@ __global__ void __launch_bounds__(256) wino_f32_stream(ConvArgs a) {
     } else {
       int live;
       const int cg = column_tile_of<KW>(a, Tp, cw, live);
-      decode_tile(a, (Tp % (a.kgroups / KW)) * KW + kw, cg, lane, wp);
+      decode_tile(a, (Tp / a.colblocks) * KW + kw, cg, lane, wp);
     }
   };
   decode_p();
@@ -645,7 +648,7 @@ __global__ void __launch_bounds__(256) wino_f32_stream(ConvArgs a) {
       if (++cq == chunks) {
         cq = 0;
         ++Tq;
-        kgq = ((Tq % (a.kgroups / KW)) * KW) + kw;
+        kgq = (Tq / a.colblocks) * KW + kw;
       }
     }
   };

@@ -64,14 +64,13 @@ __global__ void __launch_bounds__(256) wino_h16_fused_lds(ConvArgs a) {
   const int kw = wave % KW, cw = wave / KW;
   const int L = logical_block();
   if (L >= a.nblocks) return;  // whole workgroup
-  const int kblocks = a.kgroups / KW;
-  const int cg_raw = (L / kblocks) * CW + cw;
+  const int cg_raw = (L % a.colblocks) * CW + cw;
   const bool live = cg_raw < a.colgroups;
   // A workgroup whose last column tile does not exist keeps those waves busy on a copy of
   // the last real one (they must take part in the barriers) and drops their stores.
   const int cg = live ? cg_raw : a.colgroups - 1;
   WaveTile w;
-  decode_tile(a, (L % kblocks) * KW + kw, cg, lane, w);
+  decode_tile(a, (L / a.colblocks) * KW + kw, cg, lane, w);
   const int nl = lane & 31, j = lane >> 5;
   const size_t HWN = (size_t)a.H * a.W * a.N;
 
