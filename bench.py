@@ -41,10 +41,10 @@ DEFAULT_WORKLOAD = "resnet_n64_c64_h56_k64"
 # HBM bytes per launch of the fused kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # (profiles/), or None where not measured yet.
 MEASURED_TRAFFIC_BYTES = {
-    "resnet_n64_c64_h56_k64": 155.4e6,
-    "resnet_n128_c128_h28_k128": 194.7e6,
-    "deep_n128_c256_h14_k256": 155.9e6,
-    "deep_n128_c512_h7_k512": 178.0e6,
+    "resnet_n64_c64_h56_k64": 265.1e6,
+    "resnet_n128_c128_h28_k128": 267.0e6,
+    "deep_n128_c256_h14_k256": 255.4e6,
+    "deep_n128_c512_h7_k512": 116.7e6,
 }
 
 
