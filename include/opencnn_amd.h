@@ -2,8 +2,10 @@
  * opencnn_amd — C ABI of the MI355X (gfx950) Winograd F(2x2,3x3) forward convolution.
  *
  * Plain C: pointers and sizes only.  Every device pointer is memory the CALLER
- * allocated on the current HIP device; the library allocates nothing and keeps no
- * state between calls except the stream selected with opencnn_set_stream().
+ * allocated on the current HIP device; the library allocates nothing.  Its state between
+ * calls is the process-wide settings of the opencnn_set_* calls below (stream, kernel variant,
+ * balanced split, operand precision) and 8 KB of static device memory that the balanced split
+ * uses to hand tiles over between workgroups (zero between launches).
  * All entry points return a hipError_t value as int (0 == hipSuccess); launches are
  * asynchronous on the selected stream, exactly like the reference, which returns
  * cudaGetLastError() right after its two launches
@@ -13,8 +15,10 @@
  *   input   CHWN  [in_c][in_h][in_w][in_n]      src/openCNN_winograd.cu:149-150,230
  *   filter  CRSK  [filt_c][3][3][filt_k]        src/openCNN_winograd.cu:235, src/FX_m2.cu:56-57
  *   output  KHWN  [out_c][out_h][out_w][out_n]  src/store_and_transform_output_optSTS64.cuh:85-87
- *   Ww      filt_c*16*filt_k floats of caller-owned scratch, overwritten by every call
- *           (src/openCNN_winograd.cu:310-311).  Its CONTENT is the transformed filter
+ *   Ww      opencnn_workspace_bytes(filt_c, filt_k) bytes of caller-owned scratch, overwritten
+ *           by every call: filt_c*16*filt_k floats as in the reference
+ *           (src/openCNN_winograd.cu:310-311) on the shapes the reference takes, more on the
+ *           others (see opencnn_workspace_bytes).  Its CONTENT is the transformed filter
  *           U = G g G^T in an MFMA-operand order private to this library; use
  *           opencnn_filter_transform(..., OPENCNN_WW_REFERENCE) to obtain the reference's
  *           [filt_c][16][filt_k] order (src/FX_m2.cu:58-59,84).
@@ -31,7 +35,8 @@ extern "C" {
 /* Layout of the transformed-filter buffer written by opencnn_filter_transform. */
 enum {
   OPENCNN_WW_REFERENCE = 0, /* [filt_c][16][filt_k], position p = i*4+j (src/FX_m2.cu:84) */
-  OPENCNN_WW_MFMA = 1       /* [filt_k/32][filt_c/4][16][2][32][2]: what the fused kernels read */
+  OPENCNN_WW_MFMA = 1       /* [kp/32][cp/4][16][2][32][2], kp / cp = filt_k / filt_c rounded up to 32 / 8,
+                               padding zero: what the fused kernels read */
 };
 
 /* Layout of the 3x3 filters handed to the library. */
@@ -73,9 +78,12 @@ int opencnn_init(void);
  * Unlike the reference, which mis-computes silently or returns an uninitialised value
  * on shapes it does not support (src/openCNN_winograd.cu:212-218), unsupported
  * arguments return hipErrorInvalidValue and launch nothing.  Supported: filt_h ==
- * filt_w == 3, m == 2, alpha == tile_size == 4, in_n % 32 == 0, filt_k % 32 == 0,
- * in_c % 8 == 0, filt_c == in_c, out_* consistent with pad 1 / stride 1, tiles_dim ==
- * opencnn_tiles_dim(in_w), in_h == in_w, every tensor below 2^31 elements.
+ * filt_w == 3, m == 2, alpha == tile_size == 4, filt_c == in_c, out_* consistent with pad 1 /
+ * stride 1, tiles_dim == opencnn_tiles_dim(in_w), in_h == in_w, every tensor below 2^31
+ * elements.  in_n, in_c and filt_k are free: outside the reference's in_n % 32 == 0,
+ * filt_k % 64 == 0, in_c % 8 == 0 the groups are rounded up and the missing lanes, channels
+ * and filters predicated (Ww must then hold opencnn_workspace_bytes(), which is more than the
+ * reference's filt_k*filt_c*16 floats).
  */
 int convolutionForward(float *k, int in_h, int in_w, float *w, int out_h, int out_w,
                        int out_n, int out_c, float *C, float *Ww, const unsigned int n,
@@ -98,8 +106,9 @@ int convolutionForward_32x64x8(float *k, int in_h, int in_w, float *w, int out_h
  * src/openCNN_winograd.cu:286-288. */
 int opencnn_tiles_dim(int in_w);
 
-/* Size in bytes of the Ww scratch: filt_k*filt_c*16*sizeof(float), the caller-side
- * cudaMalloc at src/openCNN_winograd.cu:310-311. */
+/* Size in bytes of the Ww scratch: 16*sizeof(float) for each of filt_k (rounded up to 32) x
+ * filt_c (rounded up to 8) filters.  On the shapes the reference takes this is its caller-side
+ * cudaMalloc, filt_k*filt_c*16*sizeof(float) (src/openCNN_winograd.cu:310-311). */
 size_t opencnn_workspace_bytes(int filt_c, int filt_k);
 
 /* Stream (a hipStream_t passed as void*) used by every later call from any thread;
@@ -111,13 +120,15 @@ int opencnn_set_stream(void *stream);
  * Which fused kernel later calls launch.  The reference picks its variant at compile time
  * (-DBASE / -DOPTSTS64 / -DOPTSTS64_CMP / -DOPTLDS64, Makefile:3,8); here it is a run-time
  * switch so both can be measured in one process.
- *   OPENCNN_KERNEL_AUTO      the LDS variant when filt_k % 64 == 0 (as one continuous pipeline
- *                            over all tiles of a workgroup when the balanced split is in use),
- *                            else the register variant
+ *   OPENCNN_KERNEL_AUTO      the LDS variant when the 32-wide filter groups (filt_k / 32, rounded
+ *                            up) pair up (as one continuous pipeline over all tiles of a
+ *                            workgroup when the balanced split is in use), else the register
+ *                            variant
  *   OPENCNN_KERNEL_REGISTER  every wave transforms its own input patches; no LDS, no barriers
  *   OPENCNN_KERNEL_LDS       the waves of a workgroup that share a column tile split the input
- *                            transform and exchange it through LDS (needs filt_k % 64 == 0,
- *                            otherwise later launches return hipErrorInvalidValue)
+ *                            transform and exchange it through LDS (needs an even number of
+ *                            filter groups, otherwise later launches return
+ *                            hipErrorInvalidValue)
  */
 enum { OPENCNN_KERNEL_AUTO = 0, OPENCNN_KERNEL_REGISTER = 1, OPENCNN_KERNEL_LDS = 2 };
 int opencnn_set_kernel_variant(int variant);
@@ -139,7 +150,8 @@ int opencnn_set_balanced_split(int enable);
  * The reference's FX kernel as a call of its own (src/FX_m2.cu:51-91, launched at
  * src/convolutionForward_32x64x8.cu:274): U = G g G^T for every (c,k).
  *   w              device, filt_c*9*filt_k floats in `filter_layout`
- *   Ww             device, filt_c*16*filt_k floats, written in `ww_layout`
+ *   Ww             device, written in `ww_layout`: filt_c*16*filt_k floats for
+ *                  OPENCNN_WW_REFERENCE, opencnn_workspace_bytes() for OPENCNN_WW_MFMA
  * OPENCNN_WW_REFERENCE output is bit-identical to the reference's arithmetic order
  * (only additions and multiplications by 0.5).
  */

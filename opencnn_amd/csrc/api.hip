@@ -50,17 +50,24 @@ int fail(const char* what) {
 
 constexpr long long kMaxElems = (1LL << 31) - 1;
 
+// Filters / channels the transformed filter is padded to (whole MFMA groups and chunks).
+long long padded_k(int filt_k) { return ((long long)filt_k + 31) / 32 * 32; }
+long long padded_c(int filt_c) { return ((long long)filt_c + 7) / 8 * 8; }
+
+// Shapes the reference takes (its BN = 32, BK = 64 halves, BC = 8 tiling); the others run on
+// rounded-up groups with predicated lanes.
+bool ragged_shape(int in_n, int in_c, int filt_k) {
+  return in_n % 32 != 0 || filt_k % 32 != 0 || in_c % 8 != 0;
+}
+
 int check_filter_shape(int filt_k, int filt_c) {
   REQUIRE(filt_k > 0 && filt_c > 0);
-  REQUIRE(filt_k % 32 == 0);
-  REQUIRE(filt_c % 8 == 0);
-  REQUIRE((long long)filt_k * filt_c * 16 <= kMaxElems / 4);  // Ww byte offsets stay below 2^31
+  REQUIRE(padded_k(filt_k) * padded_c(filt_c) * 16 <= kMaxElems / 4);  // Ww byte offsets stay below 2^31
   return 0;
 }
 
 int check_conv_shape(int in_n, int in_c, int in_h, int in_w, int filt_k) {
   REQUIRE(in_n > 0 && in_c > 0 && in_h > 0 && in_w > 0);
-  REQUIRE(in_n % 32 == 0);
   if (int e = check_filter_shape(filt_k, in_c)) return e;
   REQUIRE((long long)in_n * in_c * in_h * in_w <= kMaxElems);
   REQUIRE((long long)in_n * filt_k * in_h * in_w <= kMaxElems);
@@ -78,6 +85,7 @@ int launch_fx(const float* w, float* Ww, int filt_k, int filt_c, int filter_layo
   const int precision = g_precision.load();
   if (ww_layout == OPENCNN_WW_MFMA && precision != OPENCNN_F32) {
     REQUIRE(filt_c % 16 == 0);
+    REQUIRE(filt_k % 32 == 0);
     dim3 grid((filt_k + 127) / 128, filt_c / 16), block(256);
     uint4* out = reinterpret_cast<uint4*>(Ww);
     if (precision == OPENCNN_F16) {
@@ -100,7 +108,7 @@ int launch_fx(const float* w, float* Ww, int filt_k, int filt_c, int filter_layo
     else
       opencnn::fx_reference_layout<false><<<grid, block, 0, st>>>(w, Ww, filt_k, filt_c);
   } else {
-    dim3 grid((filt_k + 127) / 128, filt_c / 4), block(256);
+    dim3 grid((filt_k + 127) / 128, (unsigned)(padded_c(filt_c) / 4)), block(256);
     if (kcrs)
       opencnn::fx_mfma_layout<true><<<grid, block, 0, st>>>(w, Ww, filt_k, filt_c);
     else
@@ -133,12 +141,15 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   a.K = filt_k;
   a.tiles_h = (in_h + 1) / 2;
   a.tiles_w = (in_w + 1) / 2;
-  a.ngroups = in_n / 32;
+  a.ngroups = (in_n + 31) / 32;
+  REQUIRE((long long)a.tiles_h * a.tiles_w * a.ngroups <= kMaxElems / 8);
   a.colgroups = a.tiles_h * a.tiles_w * a.ngroups;
-  a.kgroups = filt_k / 32;
+  a.kgroups = (filt_k + 31) / 32;
+  const bool ragged = ragged_shape(in_n, in_c, filt_k);
   const int precision = g_precision.load();
   if (precision != OPENCNN_F32) {
     // fp16 / bf16 GEMM operands: 16-channel chunks, LDS kernel only
+    REQUIRE(in_n % 32 == 0);
     REQUIRE(in_c % 16 == 0);
     REQUIRE(filt_k % 64 == 0);
     REQUIRE((long long)in_n * in_h * in_w * 4 * 4 <= kMaxElems);  // four-channel window in bytes
@@ -168,10 +179,16 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
     }
     return (int)hipGetLastError();
   }
-  // Waves per workgroup that share one column tile (and split its input transform).
+  // Waves per workgroup that share one column tile (and split its input transform).  A
+  // ragged shape runs the LDS kernel when its (rounded-up) filter groups fill whole workgroups.
   int kw = 1;
   const int variant = g_variant.load();
-  if (variant != OPENCNN_KERNEL_REGISTER) kw = filt_k % 128 == 0 ? 4 : (filt_k % 64 == 0 ? 2 : 1);
+  if (variant != OPENCNN_KERNEL_REGISTER) {
+    if (!ragged)
+      kw = filt_k % 128 == 0 ? 4 : (filt_k % 64 == 0 ? 2 : 1);
+    else
+      kw = a.kgroups % 4 == 0 ? 4 : (a.kgroups % 2 == 0 ? 2 : 1);
+  }
   if (variant == OPENCNN_KERNEL_LDS) REQUIRE(kw > 1);
   const int cw = 4 / kw;
   const long long colblocks = (a.colgroups + cw - 1) / cw;
@@ -183,11 +200,21 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   dim3 grid(per_xcd * 8), block(256);
   const size_t lds_bytes = (size_t)cw * 2 * 4 * 16 * 64 * sizeof(float);
   if (kw == 1) {
-    opencnn::wino_f32_fused<<<grid, block, 0, st>>>(a);
+    if (ragged)
+      opencnn::wino_f32_fused<true><<<grid, block, 0, st>>>(a);
+    else
+      opencnn::wino_f32_fused<false><<<grid, block, 0, st>>>(a);
     return (int)hipGetLastError();
   }
   // More tiles than CUs and not a whole number of rounds: one persistent workgroup per CU,
   // the chunk-units split evenly (every tile then has at most two contributors).
+  if (ragged) {
+    if (kw == 4)
+      opencnn::wino_f32_fused_lds<4, false, true><<<grid, block, lds_bytes, st>>>(a);
+    else
+      opencnn::wino_f32_fused_lds<2, false, true><<<grid, block, lds_bytes, st>>>(a);
+    return (int)hipGetLastError();
+  }
   int cus = 0;
   if (int e = compute_units(&cus)) return e;
   const bool balanced = g_balance.load() != 0 && a.nblocks > cus && a.nblocks % cus != 0 &&
@@ -245,7 +272,7 @@ int opencnn_tiles_dim(int in_w) {
 
 size_t opencnn_workspace_bytes(int filt_c, int filt_k) {
   if (filt_c <= 0 || filt_k <= 0) return 0;
-  return (size_t)filt_c * (size_t)filt_k * 16 * sizeof(float);
+  return (size_t)padded_c(filt_c) * (size_t)padded_k(filt_k) * 16 * sizeof(float);
 }
 
 int opencnn_set_stream(void* stream) {

@@ -41,9 +41,9 @@ struct ConvArgs {
   float* y;          // KHWN
   int N, C, H, W, K;
   int tiles_h, tiles_w;  // 2x2 output tiles per image column / row
-  int ngroups;           // N / 32
+  int ngroups;           // ceil(N / 32)
   int colgroups;         // tiles_h * tiles_w * ngroups   (wave-level column tiles)
-  int kgroups;           // K / 32
+  int kgroups;           // ceil(K / 32)
   int nblocks;           // workgroup tiles: filter blocks x column blocks
   int colblocks;         // column blocks; workgroup tile T = filter block T / colblocks,
                          // column block T % colblocks (LDS kernels): an XCD's contiguous
@@ -103,6 +103,11 @@ struct WaveTile {
   int voff[16];  // byte offset of patch element (i,j) in a two-channel slab, or kOutOfRange
 };
 
+// RAGGED (here and below) = shapes outside the reference's N % 32 == 0, K % 32 == 0,
+// C % 8 == 0: the groups are rounded up, lanes whose batch element does not exist read zeros
+// and store nothing, channels past C read zeros on both operands, filters past K are zero
+// in the transformed filter and are not stored.
+template <bool RAGGED = false>
 __device__ __forceinline__ void decode_tile(const ConvArgs& a, int kg, int cg, int lane, WaveTile& w) {
   const int tile = cg / a.ngroups;
   w.kg = kg;
@@ -117,7 +122,8 @@ __device__ __forceinline__ void decode_tile(const ConvArgs& a, int kg, int cg, i
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int hh = 2 * w.ty - 1 + i, ww = 2 * w.tx - 1 + j;
-      const bool ok = hh >= 0 && hh < a.H && ww >= 0 && ww < a.W;
+      const bool ok = hh >= 0 && hh < a.H && ww >= 0 && ww < a.W &&
+                      (!RAGGED || w.ng * 32 + w.nl < a.N);
       w.voff[i * 4 + j] =
           ok ? (int)(((size_t)w.hsel * HW + (size_t)hh * a.W + ww) * a.N + w.ng * 32 + w.nl) * 4
              : kOutOfRange;
@@ -127,20 +133,33 @@ __device__ __forceinline__ void decode_tile(const ConvArgs& a, int kg, int cg, i
 
 // 4x4 patch of MFMA step `step` (channels 2*step + hsel); steps past the end reload the last
 // slab (the data is never used; this keeps the pipeline free of branches).
+// RAGGED: the slab ends with the tensor (an odd C leaves one channel in the last slab) and
+// steps past the end read zeros, because the padded steps of the last chunk ARE multiplied.
+template <bool RAGGED = false>
 __device__ __forceinline__ void load_patch(const ConvArgs& a, const WaveTile& w, float (&d)[16], int step) {
-  const int S = a.C >> 1;
   const size_t HWN = (size_t)a.H * a.W * a.N;
-  const int st = step < S ? step : S - 1;
-  __amdgpu_buffer_rsrc_t r = make_rsrc(a.x + (size_t)st * 2 * HWN, (unsigned)(2 * HWN * sizeof(float)));
+  int st, channels;
+  if (RAGGED) {
+    const int S = (a.C + 1) >> 1;
+    st = step < S ? step : S - 1;
+    channels = step < S ? (a.C - 2 * st < 2 ? a.C - 2 * st : 2) : 0;
+  } else {
+    const int S = a.C >> 1;
+    st = step < S ? step : S - 1;
+    channels = 2;
+  }
+  __amdgpu_buffer_rsrc_t r = make_rsrc(a.x + (size_t)st * 2 * HWN, (unsigned)(channels * HWN * sizeof(float)));
 #pragma unroll
   for (int e = 0; e < 16; ++e)
     d[e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, w.voff[e], 0, 0));
 }
 
 // A operands of filter quad `quad` (channels 4*quad .. 4*quad+3) for all 16 positions.
+template <bool RAGGED = false>
 __device__ __forceinline__ void load_u(const ConvArgs& a, const WaveTile& w, int lane, v2f (&u)[16], int quad) {
-  const int Q = a.C >> 2;
-  const __amdgpu_buffer_rsrc_t ru = make_rsrc(a.usw, (unsigned)((size_t)a.C * 16 * a.K * sizeof(float)));
+  const int Q = RAGGED ? ((a.C + 7) >> 3) * 2 : a.C >> 2;
+  const int Kp = RAGGED ? (a.K + 31) & ~31 : a.K;
+  const __amdgpu_buffer_rsrc_t ru = make_rsrc(a.usw, (unsigned)((size_t)Q * 4 * 16 * Kp * sizeof(float)));
   const int qd = quad < Q ? quad : Q - 1;
   const int soff = (w.kg * Q + qd) * (16 * 64 * 8);
 #pragma unroll
@@ -164,7 +183,7 @@ __device__ __forceinline__ void store_through(float* p, float v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
-template <StoreMode MODE>
+template <StoreMode MODE, bool RAGGED = false>
 __device__ __forceinline__ void store_tile(const ConvArgs& a, const WaveTile& w, const v16f (&acc)[16]) {
   const size_t HWN = (size_t)a.H * a.W * a.N;
   const bool row1 = 2 * w.ty + 1 < a.H;  // odd H: last tile row keeps only a = 0
@@ -197,6 +216,7 @@ __device__ __forceinline__ void store_tile(const ConvArgs& a, const WaveTile& w,
 #pragma unroll
       for (int q = 0; q < 4; ++q) o[q] += part[r][q];
     }
+    if (RAGGED && !(k < a.K && w.ng * 32 + w.nl < a.N)) continue;
     if (MODE == kStorePublish) {
       store_through(yk, o[0]);
       if (col1) store_through(yk + o1, o[1]);
@@ -225,7 +245,8 @@ __device__ __forceinline__ int logical_block() {
 
 // ------------------------------------------------------------------------------------------
 // Kernel A: every wave transforms its own patches (no LDS, no barriers).
-// Used when K is not a multiple of 64.
+// Used when K is not a multiple of 64, and (RAGGED) for every shape outside the reference's
+// N % 32 == 0, K % 32 == 0, C % 8 == 0.
 //
 // One MFMA step = two input channels.  Software pipeline, per step t (all in registers):
 //   first   the 32 add/sub that turn the patch of step t+1 (loaded one step ago) into the
@@ -235,6 +256,7 @@ __device__ __forceinline__ int logical_block() {
 //           (16 patch loads and, every other step, the 16 filter loads of the next quad).
 // The scheduling barriers pin that order; left alone hipcc sinks the loads down to their
 // first use to save registers, which exposes the full memory latency once per step.
+template <bool RAGGED>
 __global__ void __launch_bounds__(256) wino_f32_fused(ConvArgs a) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -243,7 +265,7 @@ __global__ void __launch_bounds__(256) wino_f32_fused(ConvArgs a) {
   const int cg = (L / a.kgroups) * 4 + wave;
   if (cg >= a.colgroups) return;  // wave-uniform; this kernel has no barriers
   WaveTile w;
-  decode_tile(a, L % a.kgroups, cg, lane, w);
+  decode_tile<RAGGED>(a, L % a.kgroups, cg, lane, w);
 
   v16f acc[16];
 #pragma unroll
@@ -256,12 +278,12 @@ __global__ void __launch_bounds__(256) wino_f32_fused(ConvArgs a) {
   float v[2][16];  // B operands: v[t&1] holds the transformed patch of step t
 
   // prologue: patch 0 -> v[0]; patch 1 in flight in d[1]; quad 0 in u[0]
-  load_u(a, w, lane, u[0], 0);
-  load_patch(a, w, d[0], 0);
-  load_patch(a, w, d[1], 1);
+  load_u<RAGGED>(a, w, lane, u[0], 0);
+  load_patch<RAGGED>(a, w, d[0], 0);
+  load_patch<RAGGED>(a, w, d[1], 1);
   input_transform(d[0], v[0]);
 
-  const int octs = a.C >> 3;
+  const int octs = RAGGED ? (a.C + 7) >> 3 : a.C >> 3;
   for (int oct = 0; oct < octs; ++oct) {
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
@@ -274,9 +296,9 @@ __global__ void __launch_bounds__(256) wino_f32_fused(ConvArgs a) {
       for (int p = 0; p < 16; ++p) asm volatile("" : "+v"(v[(s + 1) & 1][p]));
       __builtin_amdgcn_sched_barrier(0);
       // d[t&1] was consumed by the transform of the previous step: refill it with step t+2
-      load_patch(a, w, d[s & 1], t + 2);
-      if (s == 0) load_u(a, w, lane, u[1], 2 * oct + 1);
-      if (s == 2) load_u(a, w, lane, u[0], 2 * oct + 2);
+      load_patch<RAGGED>(a, w, d[s & 1], t + 2);
+      if (s == 0) load_u<RAGGED>(a, w, lane, u[1], 2 * oct + 1);
+      if (s == 2) load_u<RAGGED>(a, w, lane, u[0], 2 * oct + 2);
 #pragma unroll
       for (int p = 0; p < 16; ++p)
         acc[p] = __builtin_amdgcn_mfma_f32_32x32x2f32(u[s >> 1][p][s & 1], v[s & 1][p], acc[p], 0, 0, 0);
@@ -293,7 +315,7 @@ __global__ void __launch_bounds__(256) wino_f32_fused(ConvArgs a) {
       __builtin_amdgcn_sched_barrier(0);
     }
   }
-  store_tile<kStorePlain>(a, w, acc);
+  store_tile<kStorePlain, RAGGED>(a, w, acc);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -329,7 +351,7 @@ constexpr int kMaxBalancedBlocks = 1024;
 // (the second contributor clears its pair).  Launches that overlap on one GPU would share it.
 static __device__ unsigned g_split_sync[kMaxBalancedBlocks * 4 * 2];
 
-template <int KW, bool BALANCED>
+template <int KW, bool BALANCED, bool RAGGED = false>
 __global__ void __launch_bounds__(256) wino_f32_fused_lds(ConvArgs a) {
   constexpr int CW = 4 / KW;
   constexpr int SPW = 4 / KW;
@@ -338,7 +360,8 @@ __global__ void __launch_bounds__(256) wino_f32_fused_lds(ConvArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int kw = wave % KW, cw = wave / KW;
   const int L = logical_block();
-  const int chunks = a.C >> 3;
+  static_assert(!(BALANCED && RAGGED), "the merge of a cut tile is not predicated");
+  const int chunks = RAGGED ? (a.C + 7) >> 3 : a.C >> 3;
 
   // chunk-units [unit, end) of this workgroup; unit = tile * chunks + chunk
   long long unit, end;
@@ -370,7 +393,7 @@ __global__ void __launch_bounds__(256) wino_f32_fused_lds(ConvArgs a) {
     // the last real one (they must take part in the barriers) and drops their stores.
     const int cg = live ? cg_raw : a.colgroups - 1;
     WaveTile w;
-    decode_tile(a, (T / a.colblocks) * KW + kw, cg, lane, w);
+    decode_tile<RAGGED>(a, (T / a.colblocks) * KW + kw, cg, lane, w);
 
     v16f acc[16];
 #pragma unroll
@@ -393,7 +416,7 @@ __global__ void __launch_bounds__(256) wino_f32_fused_lds(ConvArgs a) {
     };
     auto load_patches = [&](int chunk) {
 #pragma unroll
-      for (int j = 0; j < SPW; ++j) load_patch(a, w, d[j], chunk * 4 + kw * SPW + j);
+      for (int j = 0; j < SPW; ++j) load_patch<RAGGED>(a, w, d[j], chunk * 4 + kw * SPW + j);
     };
     auto read_v = [&](float (&dst)[16], int buf, int step) {
 #pragma unroll
@@ -402,7 +425,7 @@ __global__ void __launch_bounds__(256) wino_f32_fused_lds(ConvArgs a) {
 
     // prologue: chunk c0 -> buf 0; chunk c0+1 patches in flight; first quad in u[0].
     // (All reads of the previous tile's LDS data precede its last barrier, so buf 0 is free.)
-    load_u(a, w, lane, u[0], 2 * c0);
+    load_u<RAGGED>(a, w, lane, u[0], 2 * c0);
     load_patches(c0);
     transform_to_lds(0);
     load_patches(c0 + 1);
@@ -416,12 +439,12 @@ __global__ void __launch_bounds__(256) wino_f32_fused_lds(ConvArgs a) {
         __builtin_amdgcn_sched_barrier(0);
         if (s == 0) transform_to_lds(buf ^ 1);  // chunk i+1: one VALU burst, then its LDS writes
         __builtin_amdgcn_sched_barrier(0);
-        if (s == 0) load_u(a, w, lane, u[1], 2 * i + 1);
-        if (s == 2) load_u(a, w, lane, u[0], 2 * i + 2);
+        if (s == 0) load_u<RAGGED>(a, w, lane, u[1], 2 * i + 1);
+        if (s == 2) load_u<RAGGED>(a, w, lane, u[0], 2 * i + 2);
         // patches of chunk i+2: 16 loads per owned step; with two owned steps (KW = 2) the second
         // batch goes behind the MFMAs of step 3, which has no other loads
-        if (s == 1) load_patch(a, w, d[0], (i + 2) * 4 + kw * SPW);
-        if (s == 3 && SPW == 2) load_patch(a, w, d[1], (i + 2) * 4 + kw * SPW + 1);
+        if (s == 1) load_patch<RAGGED>(a, w, d[0], (i + 2) * 4 + kw * SPW);
+        if (s == 3 && SPW == 2) load_patch<RAGGED>(a, w, d[1], (i + 2) * 4 + kw * SPW + 1);
         if (s < 3) read_v(v[(s + 1) & 1], buf, s + 1);
 #pragma unroll
         for (int p = 0; p < 16; ++p)
@@ -443,7 +466,7 @@ __global__ void __launch_bounds__(256) wino_f32_fused_lds(ConvArgs a) {
 
     if (!live) continue;
     if (!BALANCED || (c0 == 0 && c1 == chunks)) {
-      store_tile<kStorePlain>(a, w, acc);
+      store_tile<kStorePlain, RAGGED>(a, w, acc);
       continue;
     }
     // Partial tile: the other part belongs to the previous (c0 > 0) or next workgroup.

@@ -66,22 +66,36 @@ __global__ void __launch_bounds__(256) fx_reference_layout(const float* __restri
 // so that lane (h*32 + k32) of a wave fetches, with one 8-byte load per position p, the A
 // operand of two consecutive v_mfma_f32_32x32x2_f32 steps (channels 4q+h and 4q+2+h).
 // Thread = (k, q, h): transforms the two channels c = 4q+h and 4q+2+h and writes float2.
-// grid (ceil(K/128), C/4), block 256 = 2 h x 128 k.
+// grid (ceil(K/128), Cpad/4), block 256 = 2 h x 128 k.
+//
+// Shapes the reference does not take (K not a multiple of 32, C not a multiple of 8) are
+// padded here: the layout covers Kpad = 32*ceil(K/32) filters and Cpad = 8*ceil(C/8) channels,
+// and the filters / channels that do not exist are written as zeros, so the fused kernel needs
+// no special case in its reduction.
 template <bool KCRS>
 __global__ void __launch_bounds__(256) fx_mfma_layout(const float* __restrict__ w,
                                                       float* __restrict__ Usw, int K, int C) {
   const int h = threadIdx.x >> 7;
   const int k = blockIdx.x * 128 + (threadIdx.x & 127);
   const int q = blockIdx.y;
-  if (k >= K) return;
-  float g0[9], g1[9], U0[16], U1[16];
-  load_filter<KCRS>(w, 4 * q + h, k, C, K, g0);
-  load_filter<KCRS>(w, 4 * q + 2 + h, k, C, K, g1);
-  fx_one(g0, U0);
-  fx_one(g1, U1);
+  if (k >= ((K + 31) & ~31)) return;
+  float U0[16], U1[16];
+#pragma unroll
+  for (int p = 0; p < 16; ++p) U0[p] = U1[p] = 0.0f;
+  if (k < K) {
+    float g[9];
+    if (4 * q + h < C) {
+      load_filter<KCRS>(w, 4 * q + h, k, C, K, g);
+      fx_one(g, U0);
+    }
+    if (4 * q + 2 + h < C) {
+      load_filter<KCRS>(w, 4 * q + 2 + h, k, C, K, g);
+      fx_one(g, U1);
+    }
+  }
   const int kg = k >> 5, k32 = k & 31;
   float2* o = reinterpret_cast<float2*>(Usw) +
-              (((size_t)kg * (C >> 2) + q) * 16) * 64 + h * 32 + k32;
+              (((size_t)kg * gridDim.y + q) * 16) * 64 + h * 32 + k32;
 #pragma unroll
   for (int p = 0; p < 16; ++p) o[(size_t)p * 64] = make_float2(U0[p], U1[p]);
 }

@@ -30,6 +30,9 @@ def test_tiles_dim_and_workspace(ocn, oracle):
         assert ocn.tiles_dim(w) == oracle.tiles_dim(w) == (w + 1) // 2
     assert ocn.workspace_bytes(256, 256) == 256 * 256 * 16 * 4
     assert ocn.workspace_bytes(0, 64) == 0
+    # shapes outside the reference's tiling: filters padded to 32, channels to 8
+    assert ocn.workspace_bytes(12, 48) == 16 * 64 * 16 * 4
+    assert ocn.workspace_bytes(1, 1) == 8 * 32 * 16 * 4
 
 
 def _call(ocn, **over):
@@ -47,7 +50,7 @@ def _call(ocn, **over):
 
 
 @pytest.mark.parametrize("over", [
-    dict(N=48), dict(N=0), dict(K=48), dict(C=12), dict(C=0), dict(R=5), dict(S=1), dict(m=4),
+    dict(N=0), dict(N=-32), dict(K=0), dict(C=0), dict(R=5), dict(S=1), dict(m=4),
     dict(alpha=6), dict(tile=6), dict(H=8, W=10), dict(out_h=6), dict(out_n=64), dict(out_c=32),
     dict(filt_c=16), dict(tiles_dim=3), dict(ptr=0), dict(N=1 << 20, H=56, W=56),
 ])
@@ -60,8 +63,8 @@ def test_unsupported_arguments_are_rejected(ocn, over):
 
 def test_filter_transform_rejects_bad_arguments(ocn):
     f = ocn.lib().opencnn_filter_transform
-    assert f(0x1000, 0x1000, 48, 8, 0, 0) == 1
-    assert f(0x1000, 0x1000, 64, 12, 0, 0) == 1
+    assert f(0x1000, 0x1000, 0, 8, 0, 0) == 1
+    assert f(0x1000, 0x1000, 64, -8, 0, 0) == 1
     assert f(0x1000, 0x1000, 64, 8, 2, 0) == 1
     assert f(0x1000, 0x1000, 64, 8, 0, 2) == 1
     assert f(0, 0x1000, 64, 8, 0, 0) == 1

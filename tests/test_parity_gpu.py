@@ -87,7 +87,8 @@ def check_against_oracle(oracle, y, x, w):
 
 # ---------------------------------------------------------------- filter transform (FX)
 
-@pytest.mark.parametrize("C,K", [(8, 64), (64, 64), (128, 128), (256, 256), (512, 512), (8, 32), (24, 96)])
+@pytest.mark.parametrize("C,K", [(8, 64), (64, 64), (128, 128), (256, 256), (512, 512), (8, 32), (24, 96),
+                                 (1, 1), (3, 40), (12, 48), (21, 130)])
 def test_fx_bit_exact(ocn, oracle, torch_gpu, C, K):
     torch = torch_gpu
     print(f"fx C={C} K={K}", flush=True)
@@ -100,10 +101,14 @@ def test_fx_bit_exact(ocn, oracle, torch_gpu, C, K):
         ocn.filter_transform(wd, out, K, C, layout, ocn.WW_REFERENCE)
         torch.cuda.synchronize()
         assert np.array_equal(out.cpu().numpy().reshape(C, 16, K), want)
-        out.fill_(float("nan"))
+        # MFMA-operand order: filters padded to 32, channels to 8, the padding written as zeros
+        out = torch.full((ocn.workspace_bytes(C, K) // 4,), float("nan"), device="cuda")
         ocn.filter_transform(wd, out, K, C, layout, ocn.WW_MFMA)
         torch.cuda.synchronize()
-        assert np.array_equal(ocn.unswizzle_ww(out.cpu().numpy(), C, K), want)
+        got = out.cpu().numpy()
+        assert np.array_equal(ocn.unswizzle_ww(got, C, K), want)
+        assert not np.isnan(got).any()
+        assert np.count_nonzero(got) == np.count_nonzero(want)
 
 
 # ---------------------------------------------------------------- whole path, benchmark sizes
@@ -258,6 +263,69 @@ def test_balanced_split_matches_plain_launch(ocn, oracle, torch_gpu, N, C, H, K)
         ocn.set_balanced_split(True)
     check_against_oracle(oracle, y0, x, w)
     np.testing.assert_allclose(y1, y0, rtol=0, atol=2e-6 * np.abs(y0).max())
+
+
+# ---------------------------------------------------------------- shapes outside the reference's tiling
+
+RAGGED = [
+    # N, C, H, W, K
+    (1, 1, 1, 1, 1),        # one of everything
+    (1, 3, 9, 9, 8),        # a single image
+    (7, 5, 6, 6, 40),       # nothing aligned
+    (33, 8, 8, 8, 64),      # batch tail only
+    (48, 12, 7, 7, 64),     # batch and channel tails, odd image
+    (32, 9, 10, 10, 32),    # odd channel count only
+    (32, 8, 8, 8, 72),      # filter tail only
+    (50, 20, 13, 13, 100),
+    (64, 30, 5, 11, 136),   # H != W through the split entry points
+]
+
+
+@pytest.mark.parametrize("N,C,H,W,K", RAGGED)
+def test_shapes_outside_reference_tiling(ocn, oracle, torch_gpu, N, C, H, W, K):
+    # The reference needs N % 32 == 0, K % 64 == 0, C % 8 == 0 and mis-computes silently
+    # otherwise (src/openCNN_winograd.cu:212-218); here groups are rounded up and the lanes,
+    # channels and filters that do not exist are predicated.  Guard bands around the output
+    # catch a store from a lane that should have been off.
+    print(f"ragged N={N} C={C} H={H} W={W} K={K}", flush=True)
+    x, w = make_tensors(ocn, N, C, H, W, K, filt="uniform")
+    r = Runner(ocn, torch_gpu, x, w)
+    y = r.split()
+    assert not np.isnan(y).any(), "an output element was never written"
+    rel64, _, _ = oracle.compare(y, oracle.direct_conv_f64(x, w))
+    assert rel64 <= 1e-5, f"rel-L2 vs fp64 direct {rel64:.3e}"
+    if H == W:
+        check_against_oracle(oracle, y, x, w)
+        assert np.array_equal(r.dropin(), y)
+
+
+def test_ragged_shape_on_both_kernel_families(ocn, oracle, torch_gpu):
+    # two filter groups: the LDS kernel by default, the register kernel on request
+    print("ragged variants", flush=True)
+    x, w = make_tensors(ocn, 48, 12, 7, 7, 64, filt="uniform")
+    r = Runner(ocn, torch_gpu, x, w)
+    y_lds = r.dropin()
+    try:
+        ocn.set_kernel_variant(ocn.KERNEL_REGISTER)
+        y_reg = r.dropin()
+    finally:
+        ocn.set_kernel_variant(ocn.KERNEL_AUTO)
+    check_against_oracle(oracle, y_lds, x, w)
+    check_against_oracle(oracle, y_reg, x, w)
+
+
+def test_padded_channels_do_not_leak_non_finite_values(ocn, oracle, torch_gpu):
+    # C = 5 runs one 8-channel chunk; the three padded channels multiply zeros on BOTH operands,
+    # so an infinity in the last real channel must stay confined to the outputs it reaches
+    print("ragged inf", flush=True)
+    N, C, H, K = 32, 5, 6, 32
+    x, w = make_tensors(ocn, N, C, H, H, K, filt="uniform")
+    x[C - 1, 2, 2, 3] = np.inf
+    y = Runner(ocn, torch_gpu, x, w).split()
+    bad = ~np.isfinite(y)
+    assert bad[:, :, :, 3].any()
+    bad[:, :, :, 3] = False
+    assert not bad.any()
 
 
 # ---------------------------------------------------------------- layout shims
