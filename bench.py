@@ -86,6 +86,26 @@ class Layer:
                                      self.H, self.K, warmup=warmup, iters=iters)
 
 
+def miopen_column(torch, lay, warmup=10, iters=50):
+    """Informational only, never an oracle: ms per call of torch.nn.functional.conv2d (MIOpen's
+    own choice of fp32 algorithm) on the same layer in NCHW / KCRS, the analogue of the
+    reference bench's cuDNN column (src/openCNN_winograd.cu:449-464)."""
+    x = lay.x.permute(3, 0, 1, 2).contiguous()
+    w = lay.w.permute(3, 0, 1, 2).contiguous()
+    torch.backends.cudnn.benchmark = True  # let MIOpen search instead of taking its first guess
+    for _ in range(warmup):
+        y = torch.nn.functional.conv2d(x, w, padding=1)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    torch.cuda.synchronize()
+    ev[0].record()
+    for _ in range(iters):
+        y = torch.nn.functional.conv2d(x, w, padding=1)
+    ev[1].record()
+    torch.cuda.synchronize()
+    del y
+    return ev[0].elapsed_time(ev[1]) / iters
+
+
 def cpu_baseline(layer):
     """The oracle's fp64 direct convolution on the host cores, one warm + one timed pass."""
     from oracle import oracle
@@ -117,6 +137,8 @@ def main():
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(FP32_LAYERS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-layers", action="store_true", help="skip the per-layer table")
+    ap.add_argument("--miopen", action="store_true",
+                    help="add an informational MIOpen (torch conv2d, fp32) column to the per-layer table")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build runs on ONE GPU (a single layer on one device, no "
@@ -206,7 +228,11 @@ def main():
                     tot, mn, fx = lay.kernel_times(20, 200)
                 finally:
                     ocn.set_operand_precision(ocn.F32)
+                extra = {}
+                if args.miopen and label == "f32":
+                    extra["ms_miopen_conv2d_fp32"] = miopen_column(torch, lay)
                 rows.append({
+                    **extra,
                     "workload": name, "gemm_operands": label, "ms_per_layer": tot, "ms_fused_kernel": mn,
                     "ms_filter_transform": fx,
                     "effective_tflops": d / (tot * 1e-3) / 1e12,
