@@ -120,17 +120,30 @@ int opencnn_set_stream(void *stream);
  * Which fused kernel later calls launch.  The reference picks its variant at compile time
  * (-DBASE / -DOPTSTS64 / -DOPTSTS64_CMP / -DOPTLDS64, Makefile:3,8); here it is a run-time
  * switch so both can be measured in one process.
- *   OPENCNN_KERNEL_AUTO      the LDS variant when the 32-wide filter groups (filt_k / 32, rounded
- *                            up) pair up (as one continuous pipeline over all tiles of a
- *                            workgroup when the balanced split is in use), else the register
- *                            variant
+ *   OPENCNN_KERNEL_AUTO      the hand-scheduled assembly kernels where they apply (see
+ *                            OPENCNN_KERNEL_ASM), else what OPENCNN_KERNEL_HIP selects
  *   OPENCNN_KERNEL_REGISTER  every wave transforms its own input patches; no LDS, no barriers
  *   OPENCNN_KERNEL_LDS       the waves of a workgroup that share a column tile split the input
  *                            transform and exchange it through LDS (needs an even number of
  *                            filter groups, otherwise later launches return
  *                            hipErrorInvalidValue)
+ *   OPENCNN_KERNEL_ASM       the LDS scheme as hand-scheduled gfx950 assembly, one persistent
+ *                            launch over all (tile, 8-channel chunk) units.  Needs in_n % 32 == 0,
+ *                            in_c % 8 == 0, filt_k % 64 == 0 and a number of workgroup tiles that
+ *                            is at least the number of compute units or a multiple of 8;
+ *                            otherwise later launches return hipErrorInvalidValue
+ *   OPENCNN_KERNEL_HIP       the HIP C++ kernels only: the LDS variant when the 32-wide filter
+ *                            groups (filt_k / 32, rounded up) pair up (as one continuous pipeline
+ *                            over all tiles of a workgroup when the balanced split is in use),
+ *                            else the register variant
  */
-enum { OPENCNN_KERNEL_AUTO = 0, OPENCNN_KERNEL_REGISTER = 1, OPENCNN_KERNEL_LDS = 2 };
+enum {
+  OPENCNN_KERNEL_AUTO = 0,
+  OPENCNN_KERNEL_REGISTER = 1,
+  OPENCNN_KERNEL_LDS = 2,
+  OPENCNN_KERNEL_ASM = 3,
+  OPENCNN_KERNEL_HIP = 4
+};
 int opencnn_set_kernel_variant(int variant);
 
 /*

@@ -29,6 +29,8 @@ from .binding import (  # noqa: F401
     KERNEL_AUTO,
     KERNEL_REGISTER,
     KERNEL_LDS,
+    KERNEL_ASM,
+    KERNEL_HIP,
     synth_filter,
     synth_input,
     tiles_dim,

@@ -20,7 +20,7 @@ WW_REFERENCE, WW_MFMA = 0, 1
 FILTER_CRSK, FILTER_KCRS = 0, 1
 INPUT_CHWN, INPUT_NCHW = 0, 1
 DIST_UNIFORM, DIST_NORMAL = 0, 1
-KERNEL_AUTO, KERNEL_REGISTER, KERNEL_LDS = 0, 1, 2
+KERNEL_AUTO, KERNEL_REGISTER, KERNEL_LDS, KERNEL_ASM, KERNEL_HIP = 0, 1, 2, 3, 4
 F32, F16, BF16 = 0, 1, 2
 
 _c_int, _c_float_p, _c_void_p = ctypes.c_int, ctypes.POINTER(ctypes.c_float), ctypes.c_void_p
@@ -166,7 +166,7 @@ def set_stream(stream) -> None:
 
 
 def set_kernel_variant(variant: int) -> None:
-    """KERNEL_AUTO, KERNEL_REGISTER or KERNEL_LDS for later launches."""
+    """KERNEL_AUTO, KERNEL_REGISTER, KERNEL_LDS, KERNEL_ASM or KERNEL_HIP for later launches."""
     _check("opencnn_set_kernel_variant", lib().opencnn_set_kernel_variant(variant))
 
 

@@ -7,7 +7,9 @@
 
 #include <atomic>
 #include <cmath>
+#include <cstdint>
 #include <cstring>
+#include <mutex>
 
 #include "conv_kernel_f32.hpp"
 #include "conv_kernel_h16.hpp"
@@ -37,6 +39,60 @@ int compute_units(int* out) {
   return 0;
 }
 thread_local const char* t_last_error = "";
+
+// ---- hand-scheduled assembly kernels (gen_wino_f32_asm.py), loaded from the embedded code object
+extern "C" const char opencnn_wino_f32_asm_hsaco[];
+
+struct AsmKernels {
+  hipModule_t module = nullptr;
+  hipFunction_t kw2 = nullptr, kw4 = nullptr;
+  unsigned* split_sync = nullptr;  // device address of g_split_sync on this device
+  bool ready = false;
+};
+
+// Loaded once per device, with that device current.
+int asm_kernels(const AsmKernels** out) {
+  static AsmKernels per_device[64];
+  static std::mutex mu;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= 64) return (int)hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(mu);
+  AsmKernels& k = per_device[dev];
+  if (!k.ready) {
+    if ((e = hipModuleLoadData(&k.module, opencnn_wino_f32_asm_hsaco)) != hipSuccess) return (int)e;
+    if ((e = hipModuleGetFunction(&k.kw2, k.module, "wino_f32_asm_kw2")) != hipSuccess) return (int)e;
+    if ((e = hipModuleGetFunction(&k.kw4, k.module, "wino_f32_asm_kw4")) != hipSuccess) return (int)e;
+    if ((e = hipGetSymbolAddress(reinterpret_cast<void**>(&k.split_sync), HIP_SYMBOL(opencnn::g_split_sync))) != hipSuccess)
+      return (int)e;
+    // 64 KB of dynamic LDS for KW = 2 is the default limit exactly; nothing to raise
+    k.ready = true;
+  }
+  *out = &k;
+  return 0;
+}
+
+// Argument block of the assembly kernels (128 bytes, the layout gen_wino_f32_asm.py loads).
+struct AsmKernArgs {
+  const float* x;
+  const float* usw;
+  float* y;
+  unsigned* sync;
+  int32_t N, H, W, chunks, tiles_w, ngroups, colgroups, colblocks;
+  int32_t Q, HWN4, units_q, units_rem, usw_bytes, grid_per_xcd;
+  uint32_t m_chunks, s_chunks, m_colblocks, s_colblocks, m_ngroups, s_ngroups, m_tiles_w, s_tiles_w;
+  int32_t spare[2];
+};
+static_assert(sizeof(AsmKernArgs) == 128, "kernel argument block");
+
+// x / d == (x * m) >> s for 0 <= x < 2^31 (round-up method, 31-bit dividends).
+void magic_divisor(uint32_t d, uint32_t* m, uint32_t* s) {
+  uint32_t l = 0;
+  while ((1ull << l) < d) ++l;
+  *m = (uint32_t)(((1ull << (31 + l)) + d - 1) / d);
+  *s = 31 + l;
+}
 
 int fail(const char* what) {
   t_last_error = what;
@@ -199,6 +255,59 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   const int per_xcd = (a.nblocks + 7) / 8;
   dim3 grid(per_xcd * 8), block(256);
   const size_t lds_bytes = (size_t)cw * 2 * 4 * 16 * 64 * sizeof(float);
+  // Hand-scheduled kernels: one persistent launch whose workgroups share the (tile, chunk) units
+  // evenly.  They need whole filter blocks, a grid that divides into the 8 XCDs and at least one
+  // tile per workgroup (a tile then has at most two contributors).
+  int agrid = 0;
+  if ((variant == OPENCNN_KERNEL_ASM || variant == OPENCNN_KERNEL_AUTO) && !ragged && kw > 1 &&
+      (long long)a.nblocks * (in_c / 8) <= kMaxElems &&
+      // per-lane store offsets: four filter rows plus one image row and column, in bytes
+      ((long long)in_n * in_h * in_w * 4 + (long long)(in_w + 1) * in_n) * 4 <= kMaxElems) {
+    int cus_asm = 0;
+    if (int e = compute_units(&cus_asm)) return e;
+    if (a.nblocks >= cus_asm) {
+      if (cus_asm % 8 == 0 && cus_asm <= opencnn::kMaxBalancedBlocks &&
+          (a.nblocks % cus_asm == 0 || g_balance.load() != 0))
+        agrid = cus_asm;
+    } else if (a.nblocks % 8 == 0) {
+      agrid = a.nblocks;
+    }
+  }
+  if (variant == OPENCNN_KERNEL_ASM) REQUIRE(agrid > 0);
+  if (agrid > 0) {
+    const int chunks = in_c / 8;
+    const AsmKernels* ak = nullptr;
+    if (int e = asm_kernels(&ak)) return e;
+    AsmKernArgs ka{};
+    ka.x = in;
+    ka.usw = Ww;
+    ka.y = out;
+    ka.sync = ak->split_sync;
+    ka.N = in_n;
+    ka.H = in_h;
+    ka.W = in_w;
+    ka.chunks = chunks;
+    ka.tiles_w = a.tiles_w;
+    ka.ngroups = a.ngroups;
+    ka.colgroups = a.colgroups;
+    ka.colblocks = a.colblocks;
+    ka.Q = in_c / 4;
+    ka.HWN4 = in_n * in_h * in_w * 4;
+    const long long total = (long long)a.nblocks * chunks;
+    ka.units_q = (int32_t)(total / agrid);
+    ka.units_rem = (int32_t)(total % agrid);
+    ka.usw_bytes = (int32_t)((long long)in_c * 16 * filt_k * 4);
+    ka.grid_per_xcd = agrid / 8;
+    magic_divisor((uint32_t)chunks, &ka.m_chunks, &ka.s_chunks);
+    magic_divisor((uint32_t)a.colblocks, &ka.m_colblocks, &ka.s_colblocks);
+    magic_divisor((uint32_t)a.ngroups, &ka.m_ngroups, &ka.s_ngroups);
+    magic_divisor((uint32_t)a.tiles_w, &ka.m_tiles_w, &ka.s_tiles_w);
+    size_t ka_size = sizeof(ka);
+    void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &ka, HIP_LAUNCH_PARAM_BUFFER_SIZE, &ka_size,
+                     HIP_LAUNCH_PARAM_END};
+    return (int)hipModuleLaunchKernel(kw == 4 ? ak->kw4 : ak->kw2, (unsigned)agrid, 1, 1, 256, 1, 1,
+                                      (unsigned)lds_bytes, st, nullptr, extra);
+  }
   if (kw == 1) {
     if (ragged)
       opencnn::wino_f32_fused<true><<<grid, block, 0, st>>>(a);
@@ -282,7 +391,8 @@ int opencnn_set_stream(void* stream) {
 
 int opencnn_set_kernel_variant(int variant) {
   REQUIRE(variant == OPENCNN_KERNEL_AUTO || variant == OPENCNN_KERNEL_REGISTER ||
-          variant == OPENCNN_KERNEL_LDS);
+          variant == OPENCNN_KERNEL_LDS || variant == OPENCNN_KERNEL_ASM ||
+          variant == OPENCNN_KERNEL_HIP);
   g_variant.store(variant);
   return 0;
 }

@@ -1,0 +1,700 @@
+#!/usr/bin/env python3
+"""Generator of the hand-scheduled gfx950 assembly of the fused Winograd F(2x2,3x3) kernel.
+
+Emits one kernel per KW (waves of a workgroup that share a column tile): wino_f32_asm_kw2 and
+wino_f32_asm_kw4.  Same mathematics and data layout as wino_f32_stream in
+conv_kernel_f32.hpp (which replaces the reference's Winograd_kernel,
+src/convolutionForward_32x64x8.cu:169-262); what the assembly adds is control over the things
+hipcc does not let the C++ source decide:
+
+  * all 256 arch VGPRs are assigned by hand (no spills, no copies through accumulator
+    registers), so the epilogue and the tile switch cannot disturb the inner loop;
+  * the first MFMA step of a tile starts from the constant 0 instead of zeroing 256
+    accumulator registers;
+  * the output transform stores through ONE per-row buffer descriptor and four per-lane
+    offsets (no 64-bit pointer arithmetic on the vector ALU, which the matrix pipe shares);
+  * exactly 64 store instructions per tile, so the s_waitcnt that follows can be counted
+    instead of draining the stores;
+  * a tile whose channel range is cut between two workgroups is merged by pre-loading the
+    published partial result INTO the accumulators (A^T M A is linear: the four outputs of a
+    2x2 tile are the images of the Winograd positions (0,0), -(0,3), -(3,0), (3,3)), which
+    takes the merge out of the epilogue.
+
+Kernel arguments (one 128-byte block, see KernArgs in api.hip): four pointers (input CHWN,
+transformed filter in MFMA order, output KHWN, split-merge flags) and 24 ints.
+
+Usage: gen_wino_f32_asm.py > wino_f32_asm.s
+"""
+import sys
+
+OOB = 0x80000000
+FLAGS = 0x00020000
+
+
+class Alloc:
+    def __init__(self, first, limit):
+        self.next, self.limit, self.names = first, limit, {}
+
+    def get(self, name, n=1, align=1):
+        self.next = (self.next + align - 1) // align * align
+        base = self.next
+        self.next += n
+        assert self.next <= self.limit, f"out of registers at {name}"
+        self.names[name] = (base, n)
+        return base
+
+
+def s(i, n=1):
+    return f"s{i}" if n == 1 else f"s[{i}:{i + n - 1}]"
+
+
+def v(i, n=1):
+    return f"v{i}" if n == 1 else f"v[{i}:{i + n - 1}]"
+
+
+def a(i, n=1):
+    return f"a{i}" if n == 1 else f"a[{i}:{i + n - 1}]"
+
+
+class Kernel:
+    def __init__(self, KW):
+        self.KW = KW
+        self.CW = 4 // KW
+        self.SPW = 4 // KW
+        self.lines = []
+        self.nlabel = 0
+        self.name = f"wino_f32_asm_kw{KW}"
+        self.alloc()
+
+    # ------------------------------------------------------------------ helpers
+    def e(self, text):
+        self.lines.append("\t" + text)
+
+    def label(self, name):
+        self.lines.append(f"{name}:")
+
+    def newlabel(self, hint):
+        self.nlabel += 1
+        return f".L{self.name}_{hint}_{self.nlabel}"
+
+    def comment(self, text):
+        self.lines.append(f"\t; {text}")
+
+    # ------------------------------------------------------------------ registers
+    def alloc(self):
+        S = Alloc(4, 100)
+        self.sPtr = 8      # s[8:15]: x, usw, y, sync
+        self.sInt = 16     # s[16:39]: the 24 ints
+        S.next = 40
+        names = ["N", "H", "W", "Chunks", "TilesW", "Ngroups", "Colgroups", "Colblocks", "Q", "HWN4",
+                 "UnitsQ", "UnitsRem", "UswBytes", "GridPerXcd", "Mch", "Sch", "Mcb", "Scb", "Mng",
+                 "Sng", "Mtw", "Stw", "Spare0", "Spare1"]
+        self.S = {n: self.sInt + i for i, n in enumerate(names)}
+        self.S.update(X=8, U=10, Y=12, Sync=14)
+        for n in ["L", "Kw", "Cw", "Wave", "Begin", "Nunits", "G", "Tp", "Cp", "Tq", "Cq", "Tm", "Cm",
+                  "SegEnd", "Kind", "KgM", "KgQ", "ColStep", "RowStep", "Slab", "UoffM", "UoffQ",
+                  "Dkb", "Dlive", "Dng", "Dty", "Dtx", "RowOk", "Spin", "KwSpw"]:
+            self.S[n] = S.get(n)
+        self.S["RsrcX"] = S.get("RsrcX", 4, 4)
+        self.S["RsrcU"] = S.get("RsrcU", 4, 4)
+        self.S["RsrcY"] = S.get("RsrcY", 4, 4)
+        self.S["Yt"] = S.get("Yt", 2, 2)
+        self.S["Fl"] = S.get("Fl", 2, 2)
+        self.S["T"] = S.get("T", 8, 2)  # temporaries T0..T7 (T6:T7 = division pair)
+        self.sgpr_count = S.next
+
+        V = Alloc(1, 256)
+        self.V = {}
+        for n, cnt, al in [("Lane", 1, 1), ("LaneX", 1, 1), ("Lane8", 1, 1), ("Lane8b", 1, 1),
+                           ("Lds", 1, 1), ("LdsWr", 1, 1), ("Zero", 1, 1), ("One", 1, 1), ("Tmp", 4, 1),
+                           ("Off", 4, 1), ("Eff", 4, 1), ("VOFF", 16, 1),
+                           ("U0", 32, 2), ("U1", 32, 2), ("D0", 16, 1), ("D1", 16, 1),
+                           ("VA", 16, 2), ("VB", 16, 2), ("T", 16, 2), ("TO", 16, 2), ("MPX", 16, 1)]:
+            if n == "D1" and self.SPW == 1:
+                continue
+            self.V[n] = V.get(n, cnt, al)
+        self.vgpr_count = V.next
+        # the 64 registers that receive a published partial tile (dead at a chunk boundary)
+        self.MP = ([self.V["T"] + i for i in range(16)] + [self.V["TO"] + i for i in range(16)] +
+                   [self.V["VB"] + i for i in range(16)] + [self.V["MPX"] + i for i in range(16)])
+
+    def sr(self, name, n=1):
+        return s(self.S[name], n)
+
+    def t(self, i):
+        return s(self.S["T"] + i)
+
+    def vr(self, name, i=0, n=1):
+        return v(self.V[name] + i, n)
+
+    # ------------------------------------------------------------------ scalar pieces
+    def div(self, dst, x, m, sh):
+        """dst = x / d for x < 2^31, with (m, sh) = (ceil(2^sh / d), 31 + ceil(log2 d))."""
+        t6, t7 = self.S["T"] + 6, self.S["T"] + 7
+        self.e(f"s_mul_hi_u32 {s(t7)}, {x}, {m}")
+        self.e(f"s_mul_i32 {s(t6)}, {x}, {m}")
+        self.e(f"s_lshr_b64 {s(t6, 2)}, {s(t6, 2)}, {sh}")
+        self.e(f"s_mov_b32 {dst}, {s(t6)}")
+
+    def decode(self, T):
+        """Workgroup tile T -> Dkb (filter block), Dlive, Dng, Dty, Dtx of this wave's column tile."""
+        t = self.t
+        self.div(self.sr("Dkb"), T, self.sr("Mcb"), self.sr("Scb"))
+        self.e(f"s_mul_i32 {t(0)}, {self.sr('Dkb')}, {self.sr('Colblocks')}")
+        self.e(f"s_sub_u32 {t(0)}, {T}, {t(0)}")  # column block
+        if self.CW == 2:
+            self.e(f"s_lshl_b32 {t(0)}, {t(0)}, 1")
+            self.e(f"s_add_u32 {t(0)}, {t(0)}, {self.sr('Cw')}")
+        self.e(f"s_sub_u32 {t(1)}, {self.sr('Colgroups')}, 1")
+        self.e(f"s_cmp_lt_u32 {t(0)}, {self.sr('Colgroups')}")
+        self.e(f"s_cselect_b32 {self.sr('Dlive')}, 1, 0")
+        self.e(f"s_cselect_b32 {t(0)}, {t(0)}, {t(1)}")  # a missing column tile works on the last real one
+        self.div(t(2), t(0), self.sr("Mng"), self.sr("Sng"))  # spatial tile
+        self.e(f"s_mul_i32 {t(3)}, {t(2)}, {self.sr('Ngroups')}")
+        self.e(f"s_sub_u32 {self.sr('Dng')}, {t(0)}, {t(3)}")
+        self.div(self.sr("Dty"), t(2), self.sr("Mtw"), self.sr("Stw"))
+        self.e(f"s_mul_i32 {t(3)}, {self.sr('Dty')}, {self.sr('TilesW')}")
+        self.e(f"s_sub_u32 {self.sr('Dtx')}, {t(2)}, {t(3)}")
+
+    def patch_offsets(self):
+        """Per-lane byte offsets of the 16 patch elements of the tile in D* (P cursor), relative to
+        a two-channel slab; elements in the zero padding get an offset no num_records reaches."""
+        t = self.t
+        self.e(f"s_lshl_b32 {t(0)}, {self.sr('Dty')}, 1")
+        self.e(f"s_sub_i32 {t(0)}, {t(0)}, 1")  # first patch row
+        self.e(f"s_lshl_b32 {t(1)}, {self.sr('Dtx')}, 1")
+        self.e(f"s_sub_i32 {t(1)}, {t(1)}, 1")  # first patch column
+        self.e(f"s_mul_i32 {t(2)}, {t(0)}, {self.sr('RowStep')}")
+        self.e(f"s_mul_i32 {t(3)}, {t(1)}, {self.sr('ColStep')}")
+        self.e(f"s_add_i32 {t(2)}, {t(2)}, {t(3)}")
+        self.e(f"s_lshl_b32 {t(3)}, {self.sr('Dng')}, 7")
+        self.e(f"s_add_i32 {t(2)}, {t(2)}, {t(3)}")  # byte offset of element (0,0), may be negative
+        for i in range(4):
+            self.e(f"s_add_i32 {t(4)}, {t(0)}, {i}")
+            self.e(f"s_cmp_lt_u32 {t(4)}, {self.sr('H')}")  # unsigned: also rejects -1
+            self.e(f"s_cselect_b32 {self.sr('RowOk')}, 1, 0")
+            self.e(f"s_mov_b32 {t(3)}, {t(2)}")
+            for j in range(4):
+                self.e(f"s_add_i32 {t(4)}, {t(1)}, {j}")
+                self.e(f"s_cmp_lt_u32 {t(4)}, {self.sr('W')}")
+                self.e(f"s_cselect_b32 {t(4)}, {self.sr('RowOk')}, 0")
+                self.e(f"s_cmp_lg_u32 {t(4)}, 0")
+                self.e(f"s_cselect_b32 {t(5)}, {t(3)}, 0x{OOB:x}")
+                self.e(f"v_add_u32 {self.vr('VOFF', i * 4 + j)}, {t(5)}, {self.vr('LaneX')}")
+                if j < 3:
+                    self.e(f"s_add_i32 {t(3)}, {t(3)}, {self.sr('ColStep')}")
+            if i < 3:
+                self.e(f"s_add_i32 {t(2)}, {t(2)}, {self.sr('RowStep')}")
+
+    def slab_descriptor(self, j):
+        """RsrcX = the two-channel slab of MFMA step Cp*4 + kw*SPW + j."""
+        t = self.t
+        self.e(f"s_lshl_b32 {t(0)}, {self.sr('Cp')}, 2")
+        self.e(f"s_add_u32 {t(0)}, {t(0)}, {self.sr('KwSpw')}")
+        if j:
+            self.e(f"s_add_u32 {t(0)}, {t(0)}, {j}")
+        self.e(f"s_mul_hi_u32 {t(1)}, {t(0)}, {self.sr('Slab')}")
+        self.e(f"s_mul_i32 {t(0)}, {t(0)}, {self.sr('Slab')}")
+        rx = self.S["RsrcX"]
+        self.e(f"s_add_u32 {s(rx)}, {s(self.S['X'])}, {t(0)}")
+        self.e(f"s_addc_u32 {s(rx + 1)}, {s(self.S['X'] + 1)}, {t(1)}")
+
+    def u_offset(self, dst, kg, c, second):
+        """dst = byte offset of filter quad 2*c (+1) of filter group kg in the MFMA-order Ww."""
+        t = self.t
+        self.e(f"s_mul_i32 {t(0)}, {kg}, {self.sr('Q')}")
+        self.e(f"s_lshl_b32 {t(1)}, {c}, 1")
+        self.e(f"s_add_u32 {t(0)}, {t(0)}, {t(1)}")
+        if second:
+            self.e(f"s_add_u32 {t(0)}, {t(0)}, 1")
+        self.e(f"s_lshl_b32 {dst}, {t(0)}, 13")
+
+    def m_tile_setup(self):
+        """After decode(Tm): KgM, the four store offsets of this tile, the address of its first row."""
+        t = self.t
+        self.e(f"s_lshl_b32 {t(0)}, {self.sr('Dkb')}, {self.KW.bit_length() - 1}")
+        self.e(f"s_add_u32 {self.sr('KgM')}, {t(0)}, {self.sr('Kw')}")
+        # validity of the four outputs (odd H / W: the last tile row / column keeps one)
+        self.e(f"s_lshl_b32 {t(0)}, {self.sr('Dty')}, 1")
+        self.e(f"s_add_u32 {t(0)}, {t(0)}, 1")
+        self.e(f"s_cmp_lt_u32 {t(0)}, {self.sr('H')}")
+        self.e(f"s_cselect_b32 {t(0)}, {self.sr('Dlive')}, 0")  # row 1 stored
+        self.e(f"s_lshl_b32 {t(1)}, {self.sr('Dtx')}, 1")
+        self.e(f"s_add_u32 {t(1)}, {t(1)}, 1")
+        self.e(f"s_cmp_lt_u32 {t(1)}, {self.sr('W')}")
+        self.e(f"s_cselect_b32 {t(1)}, {self.sr('Dlive')}, 0")  # column 1 stored
+        self.e(f"s_and_b32 {t(2)}, {t(0)}, {t(1)}")
+        for q, ok in enumerate([self.sr("Dlive"), t(1), t(0), t(2)]):
+            self.e(f"s_cmp_lg_u32 {ok}, 0")
+            self.e(f"s_cselect_b32 {t(3)}, 0, 0x{OOB:x}")
+            self.e(f"v_or_b32 {self.vr('Eff', q)}, {t(3)}, {self.vr('Off', q)}")
+        # first row of the tile: y + kg*32*HWN4 + ((2ty*W + 2tx)*N + ng*32)*4
+        yt = self.S["Yt"]
+        self.e(f"s_lshl_b32 {t(0)}, {self.sr('KgM')}, 5")
+        self.e(f"s_mul_hi_u32 {t(1)}, {t(0)}, {self.sr('HWN4')}")
+        self.e(f"s_mul_i32 {t(0)}, {t(0)}, {self.sr('HWN4')}")
+        self.e(f"s_add_u32 {s(yt)}, {s(self.S['Y'])}, {t(0)}")
+        self.e(f"s_addc_u32 {s(yt + 1)}, {s(self.S['Y'] + 1)}, {t(1)}")
+        self.e(f"s_mul_i32 {t(0)}, {self.sr('Dty')}, {self.sr('RowStep')}")
+        self.e(f"s_mul_i32 {t(1)}, {self.sr('Dtx')}, {self.sr('ColStep')}")
+        self.e(f"s_add_u32 {t(0)}, {t(0)}, {t(1)}")
+        self.e(f"s_lshl_b32 {t(0)}, {t(0)}, 1")
+        self.e(f"s_lshl_b32 {t(1)}, {self.sr('Dng')}, 7")
+        self.e(f"s_add_u32 {t(0)}, {t(0)}, {t(1)}")
+        self.e(f"s_add_u32 {s(yt)}, {s(yt)}, {t(0)}")
+        self.e(f"s_addc_u32 {s(yt + 1)}, {s(yt + 1)}, 0")
+
+    # ------------------------------------------------------------------ vector pieces
+    def load_u(self, dst, p, soff):
+        lane = self.vr("Lane8") if p < 8 else self.vr("Lane8b")
+        self.e(f"buffer_load_dwordx2 {self.vr(dst, 2 * p, 2)}, {lane}, {self.sr('RsrcU', 4)}, {soff} offen offset:{(p % 8) * 512}")
+
+    def load_patch(self, dst, p):
+        self.e(f"buffer_load_dword {self.vr(dst, p)}, {self.vr('VOFF', p)}, {self.sr('RsrcX', 4)}, 0 offen")
+
+    def read_v(self, dst, step, p):
+        """Two B operands (positions p, p+1) of MFMA step `step` from the read buffer."""
+        self.e(f"ds_read2st64_b32 {self.vr(dst, p, 2)}, {self.vr('Lds')} offset0:{step * 16 + p} offset1:{step * 16 + p + 1}")
+
+    def transform(self, src, j):
+        """V = B^T d B of one patch (columns first, then rows, the order of
+        src/convolutionForward_32x64x8.cu:59-80), written to the write buffer as owned step j."""
+        d = lambda i: self.vr(src, i)
+        t = lambda i: self.vr("T", i)
+        o = lambda i: self.vr("TO", i)
+        for c in range(4):
+            self.e(f"v_sub_f32 {t(c)}, {d(c)}, {d(8 + c)}")
+            self.e(f"v_add_f32 {t(4 + c)}, {d(4 + c)}, {d(8 + c)}")
+            self.e(f"v_sub_f32 {t(8 + c)}, {d(8 + c)}, {d(4 + c)}")
+            self.e(f"v_sub_f32 {t(12 + c)}, {d(4 + c)}, {d(12 + c)}")
+        for r in range(4):
+            self.e(f"v_sub_f32 {o(4 * r)}, {t(4 * r)}, {t(4 * r + 2)}")
+            self.e(f"v_add_f32 {o(4 * r + 1)}, {t(4 * r + 1)}, {t(4 * r + 2)}")
+            self.e(f"v_sub_f32 {o(4 * r + 2)}, {t(4 * r + 2)}, {t(4 * r + 1)}")
+            self.e(f"v_sub_f32 {o(4 * r + 3)}, {t(4 * r + 1)}, {t(4 * r + 3)}")
+        for p in range(0, 16, 2):
+            self.e(f"ds_write2st64_b32 {self.vr('LdsWr')}, {o(p)}, {o(p + 1)} offset0:{j * 16 + p} offset1:{j * 16 + p + 1}")
+
+    def mfma_step(self, step, first, vmem):
+        """16 MFMAs of one step; behind MFMA p: vmem(p) (one global load or nothing) and, for
+        p < 8, the LDS read of two B operands of the next step."""
+        usrc = "U0" if step < 2 else "U1"
+        vsrc = "VA" if step % 2 == 0 else "VB"
+        vnext = "VB" if step % 2 == 0 else "VA"
+        for p in range(16):
+            c = "0" if (first and step == 0) else a(16 * p, 16)
+            self.e(f"v_mfma_f32_32x32x2_f32 {a(16 * p, 16)}, {self.vr(usrc, 2 * p + (step & 1))}, {self.vr(vsrc, p)}, {c}")
+            if vmem:
+                vmem(p)
+            if step < 3 and p < 8:
+                self.read_v(vnext, step + 1, 2 * p)
+
+    def end_of_chunk(self):
+        """All LDS traffic of this wave done, workgroup barrier, swap the buffers, fetch the first
+        B operands of the next chunk."""
+        self.e("s_waitcnt lgkmcnt(0)")
+        self.e("s_barrier")
+        self.e(f"v_xor_b32 {self.vr('Lds')}, 0x4000, {self.vr('Lds')}")
+        self.e(f"v_xor_b32 {self.vr('LdsWr')}, 0x4000, {self.vr('LdsWr')}")
+        for p in range(0, 16, 2):
+            self.read_v("VA", 0, p)
+
+    # ------------------------------------------------------------------ cursors
+    def advance_p(self):
+        skip = self.newlabel("skip_p")
+        t = self.t
+        self.e(f"s_add_u32 {t(0)}, {self.sr('G')}, 2")
+        self.e(f"s_cmp_lt_u32 {t(0)}, {self.sr('Nunits')}")
+        self.e(f"s_cbranch_scc0 {skip}")
+        self.e(f"s_add_u32 {self.sr('Cp')}, {self.sr('Cp')}, 1")
+        self.e(f"s_cmp_lt_u32 {self.sr('Cp')}, {self.sr('Chunks')}")
+        self.e(f"s_cbranch_scc1 {skip}")
+        self.e(f"s_mov_b32 {self.sr('Cp')}, 0")
+        self.e(f"s_add_u32 {self.sr('Tp')}, {self.sr('Tp')}, 1")
+        self.decode(self.sr("Tp"))
+        self.patch_offsets()
+        self.label(skip)
+
+    def advance_q(self):
+        skip = self.newlabel("skip_q")
+        t = self.t
+        self.e(f"s_add_u32 {t(0)}, {self.sr('G')}, 1")
+        self.e(f"s_cmp_lt_u32 {t(0)}, {self.sr('Nunits')}")
+        self.e(f"s_cbranch_scc0 {skip}")
+        self.e(f"s_add_u32 {self.sr('Cq')}, {self.sr('Cq')}, 1")
+        self.e(f"s_cmp_lt_u32 {self.sr('Cq')}, {self.sr('Chunks')}")
+        self.e(f"s_cbranch_scc1 {skip}")
+        self.e(f"s_mov_b32 {self.sr('Cq')}, 0")
+        self.e(f"s_add_u32 {self.sr('Tq')}, {self.sr('Tq')}, 1")
+        self.div(t(0), self.sr("Tq"), self.sr("Mcb"), self.sr("Scb"))
+        self.e(f"s_lshl_b32 {t(0)}, {t(0)}, {self.KW.bit_length() - 1}")
+        self.e(f"s_add_u32 {self.sr('KgQ')}, {t(0)}, {self.sr('Kw')}")
+        self.label(skip)
+
+    # ------------------------------------------------------------------ one chunk
+    def chunk(self, first):
+        """MFMA work of unit G (8 channels) with the loads of the units after it in its shadow.
+
+        Global loads in issue order: step 0 second filter quad of this unit (U1), step 1 patches
+        of unit G+2 (D0), step 2 first filter quad of unit G+1 (U0), step 3 (KW = 2) second
+        patch of unit G+2 (D1).  vmcnt counts in issue order, stores included; `first` = this
+        chunk follows the 64 stores of an epilogue (or a drained queue), so everything it waits
+        for is older than those stores and the counts grow by 64 (capped at the field's 63)."""
+        two = self.SPW == 2
+        wait = lambda n: self.e(f"s_waitcnt vmcnt({min(63, n + (64 if first else 0))})")
+        self.comment(f"---- chunk ({'first of a segment' if first else 'steady state'})")
+        self.advance_p()
+        self.advance_q()
+        # step 0
+        wait(32 if two else 16)  # D0 of unit G+1 has landed
+        self.transform("D0", 0)
+        self.u_offset(self.sr("UoffM"), self.sr("KgM"), self.sr("Cm"), True)
+        wait(16 if two else 0)  # U0 of this unit has landed
+        self.e("s_waitcnt lgkmcnt(8)")  # first B operands (the 8 LDS writes above may still fly)
+        self.mfma_step(0, first, lambda p: self.load_u("U1", p, self.sr("UoffM")))
+        # step 1
+        self.slab_descriptor(0)
+        self.e("s_waitcnt lgkmcnt(0)")
+        self.mfma_step(1, first, lambda p: self.load_patch("D0", p))
+        # step 2
+        if two:
+            self.e("s_waitcnt vmcnt(%d)" % (63 if first else 32))  # D1 of unit G+1 has landed
+            self.transform("D1", 1)
+        self.u_offset(self.sr("UoffQ"), self.sr("KgQ"), self.sr("Cq"), False)
+        self.e("s_waitcnt vmcnt(16)")  # U1 (step 0) has landed; only D0 (step 1) is younger
+        self.e("s_waitcnt lgkmcnt(%d)" % (8 if two else 0))
+        self.mfma_step(2, first, lambda p: self.load_u("U0", p, self.sr("UoffQ")))
+        # step 3
+        if two:
+            self.slab_descriptor(1)
+        self.e("s_waitcnt lgkmcnt(0)")
+        self.mfma_step(3, first, (lambda p: self.load_patch("D1", p)) if two else None)
+        self.end_of_chunk()
+        self.e(f"s_add_u32 {self.sr('G')}, {self.sr('G')}, 1")
+        self.e(f"s_add_u32 {self.sr('Cm')}, {self.sr('Cm')}, 1")
+
+    # ------------------------------------------------------------------ epilogue
+    def row_advance(self, r):
+        """RsrcY: filter row 8*(r/4) + r%4 -> the row of r+1 (the 4*hsel part is in the lane offset)."""
+        if r == 15:
+            return
+        ry = self.S["RsrcY"]
+        mult = 5 if r % 4 == 3 else 1
+        for _ in range(mult):
+            self.e(f"s_add_u32 {s(ry)}, {s(ry)}, {self.sr('HWN4')}")
+            self.e(f"s_addc_u32 {s(ry + 1)}, {s(ry + 1)}, 0")
+
+    def epilogue(self, through):
+        """Y = A^T M A per accumulator element (order of src/store_and_transform_output_optSTS64.cuh:29-51)
+        and the 64 stores of the tile; `through` = write past the caches (a partial tile that a
+        workgroup on another XCD will read)."""
+        pol = " sc0 sc1" if through else ""
+        ry = self.S["RsrcY"]
+        self.e(f"s_mov_b32 {s(ry)}, {s(self.S['Yt'])}")
+        self.e(f"s_mov_b32 {s(ry + 1)}, {s(self.S['Yt'] + 1)}")
+        # the last MFMAs must have written the accumulators before they are read
+        self.e("s_nop 15")
+        self.e("s_nop 15")
+        m = lambda i: self.vr("T", i)
+        for r in range(16):
+            w = lambda i: self.vr("TO", i)          # a_j: 0-3, b_j: 4-7
+            o = lambda q: self.vr("TO", 8 + 4 * (r & 1) + q)  # outputs alternate between two sets
+            for p in range(16):
+                self.e(f"v_accvgpr_read_b32 {m(p)}, {a(16 * p + r)}")
+            for j in range(4):
+                self.e(f"v_add_f32 {w(j)}, {m(j)}, {m(4 + j)}")
+                self.e(f"v_sub_f32 {w(4 + j)}, {m(4 + j)}, {m(8 + j)}")
+            for j in range(4):
+                self.e(f"v_add_f32 {w(j)}, {w(j)}, {m(8 + j)}")
+                self.e(f"v_sub_f32 {w(4 + j)}, {w(4 + j)}, {m(12 + j)}")
+            self.e(f"v_add_f32 {o(0)}, {w(0)}, {w(1)}")
+            self.e(f"v_sub_f32 {o(1)}, {w(1)}, {w(2)}")
+            self.e(f"v_add_f32 {o(2)}, {w(4)}, {w(5)}")
+            self.e(f"v_sub_f32 {o(3)}, {w(5)}, {w(6)}")
+            self.e(f"v_add_f32 {o(0)}, {o(0)}, {w(2)}")
+            self.e(f"v_sub_f32 {o(1)}, {o(1)}, {w(3)}")
+            self.e(f"v_add_f32 {o(2)}, {o(2)}, {w(6)}")
+            self.e(f"v_sub_f32 {o(3)}, {o(3)}, {w(7)}")
+            for q in range(4):
+                self.e(f"buffer_store_dword {o(q)}, {self.vr('Eff', q)}, {s(ry, 4)}, 0 offen{pol}")
+            self.row_advance(r)
+
+    def flag_address(self, previous):
+        """Fl = &flags[((L - previous) * 4 + wave) * 2 + 1]."""
+        t = self.t
+        fl = self.S["Fl"]
+        self.e(f"s_sub_u32 {t(0)}, {self.sr('L')}, {1 if previous else 0}")
+        self.e(f"s_lshl_b32 {t(0)}, {t(0)}, 2")
+        self.e(f"s_add_u32 {t(0)}, {t(0)}, {self.sr('Wave')}")
+        self.e(f"s_lshl_b32 {t(0)}, {t(0)}, 3")
+        self.e(f"s_add_u32 {t(0)}, {t(0)}, 4")
+        self.e(f"s_add_u32 {s(fl)}, {s(self.S['Sync'])}, {t(0)}")
+        self.e(f"s_addc_u32 {s(fl + 1)}, {s(self.S['Sync'] + 1)}, 0")
+
+    def store_flag(self, value_reg):
+        self.e("s_mov_b64 exec, 1")
+        self.e(f"global_store_dword {self.vr('Zero')}, {value_reg}, {s(self.S['Fl'], 2)} sc0 sc1")
+        self.e("s_mov_b64 exec, -1")
+
+    def merge_init(self):
+        """Last segment of a workgroup that ends inside a tile: the first part of that tile was
+        published by the next workgroup long ago.  Wait for its flag (bounded), read the partial
+        outputs past the caches and start the accumulators from them."""
+        t = self.t
+        self.comment("---- merge: accumulators start from the published partial tile")
+        self.flag_address(False)
+        self.e(f"s_mov_b32 {self.sr('Spin')}, 0")
+        poll, got = self.newlabel("poll"), self.newlabel("got")
+        self.label(poll)
+        self.e(f"global_load_dword {self.vr('Tmp')}, {self.vr('Zero')}, {s(self.S['Fl'], 2)} sc0 sc1")
+        self.e("s_waitcnt vmcnt(0)")
+        self.e(f"v_readfirstlane_b32 {t(0)}, {self.vr('Tmp')}")
+        self.e("s_nop 4")
+        self.e(f"s_cmp_lg_u32 {t(0)}, 0")
+        self.e(f"s_cbranch_scc1 {got}")
+        self.e(f"s_add_u32 {self.sr('Spin')}, {self.sr('Spin')}, 1")
+        self.e(f"s_cmp_lt_u32 {self.sr('Spin')}, 0x100000")
+        self.e(f"s_cbranch_scc0 {got}")  # never hang the GPU on a bug: give up and produce a wrong tile
+        self.e("s_sleep 8")
+        self.e(f"s_branch {poll}")
+        self.label(got)
+        ry = self.S["RsrcY"]
+        self.e(f"s_mov_b32 {s(ry)}, {s(self.S['Yt'])}")
+        self.e(f"s_mov_b32 {s(ry + 1)}, {s(self.S['Yt'] + 1)}")
+        for r in range(16):
+            for q in range(4):
+                self.e(f"buffer_load_dword {v(self.MP[r * 4 + q])}, {self.vr('Eff', q)}, {s(ry, 4)}, 0 offen sc0 sc1")
+            self.row_advance(r)
+        self.e("s_waitcnt vmcnt(0)")
+        # outputs (a,b) of a 2x2 tile <- positions (0,0), -(0,3), -(3,0), (3,3)
+        src = {0: (0, False), 3: (1, True), 12: (2, True), 15: (3, False)}
+        for p in range(16):
+            for r in range(16):
+                if p in src:
+                    q, neg = src[p]
+                    reg = v(self.MP[r * 4 + q])
+                    if neg:
+                        self.e(f"v_xor_b32 {reg}, 0x80000000, {reg}")
+                    self.e(f"v_accvgpr_write_b32 {a(16 * p + r)}, {reg}")
+                else:
+                    self.e(f"v_accvgpr_write_b32 {a(16 * p + r)}, 0")
+        self.store_flag(self.vr("Zero"))  # hand the flag back for the next launch
+        self.e("s_nop 15")
+        self.e("s_nop 15")
+
+    # ------------------------------------------------------------------ whole kernel
+    def body(self):
+        S, t = self.S, self.t
+        e = self.e
+        KWLOG = self.KW.bit_length() - 1
+        e(f"s_load_dwordx8 {s(8, 8)}, s[0:1], 0x0")
+        e(f"s_load_dwordx16 {s(16, 16)}, s[0:1], 0x20")
+        e(f"s_load_dwordx8 {s(32, 8)}, s[0:1], 0x60")
+        e(f"v_and_b32 {self.vr('Tmp', 1)}, 0x3ff, v0")
+        e(f"v_lshrrev_b32 {self.vr('Tmp')}, 6, {self.vr('Tmp', 1)}")
+        e(f"v_and_b32 {self.vr('Lane')}, 63, {self.vr('Tmp', 1)}")
+        e(f"v_mov_b32 {self.vr('Zero')}, 0")
+        e(f"v_mov_b32 {self.vr('One')}, 1")
+        e("s_waitcnt lgkmcnt(0)")
+        # only now: a vector instruction that writes an SGPR while scalar loads are still
+        # outstanding came back with a corrupted value on this part
+        e(f"v_readfirstlane_b32 {self.sr('Wave')}, {self.vr('Tmp')}")
+        e("s_nop 4")
+        e(f"s_and_b32 {self.sr('Kw')}, {self.sr('Wave')}, {self.KW - 1}")
+        e(f"s_lshr_b32 {self.sr('Cw')}, {self.sr('Wave')}, {KWLOG}")
+        e(f"s_mul_i32 {self.sr('KwSpw')}, {self.sr('Kw')}, {self.SPW}")
+        # logical block: workgroups are dealt round-robin to the 8 XCDs; each XCD gets a contiguous range
+        e(f"s_and_b32 {t(0)}, s2, 7")
+        e(f"s_mul_i32 {t(0)}, {t(0)}, {self.sr('GridPerXcd')}")
+        e(f"s_lshr_b32 {t(1)}, s2, 3")
+        e(f"s_add_u32 {self.sr('L')}, {t(0)}, {t(1)}")
+        # units [Begin, Begin + Nunits): the first UnitsRem blocks take one more
+        e(f"s_mul_i32 {self.sr('Begin')}, {self.sr('L')}, {self.sr('UnitsQ')}")
+        e(f"s_min_u32 {t(0)}, {self.sr('L')}, {self.sr('UnitsRem')}")
+        e(f"s_add_u32 {self.sr('Begin')}, {self.sr('Begin')}, {t(0)}")
+        e(f"s_cmp_lt_u32 {self.sr('L')}, {self.sr('UnitsRem')}")
+        e(f"s_cselect_b32 {t(0)}, 1, 0")
+        e(f"s_add_u32 {self.sr('Nunits')}, {self.sr('UnitsQ')}, {t(0)}")
+        self.div(self.sr("Tm"), self.sr("Begin"), self.sr("Mch"), self.sr("Sch"))
+        e(f"s_mul_i32 {t(0)}, {self.sr('Tm')}, {self.sr('Chunks')}")
+        e(f"s_sub_u32 {self.sr('Cm')}, {self.sr('Begin')}, {t(0)}")
+        for n in ("Tp", "Tq"):
+            e(f"s_mov_b32 {self.sr(n)}, {self.sr('Tm')}")
+        for n in ("Cp", "Cq"):
+            e(f"s_mov_b32 {self.sr(n)}, {self.sr('Cm')}")
+        e(f"s_lshl_b32 {self.sr('ColStep')}, {self.sr('N')}, 2")
+        e(f"s_mul_i32 {self.sr('RowStep')}, {self.sr('ColStep')}, {self.sr('W')}")
+        e(f"s_lshl_b32 {self.sr('Slab')}, {self.sr('HWN4')}, 1")
+        # descriptors: words 2 (num_records) and 3 (flags) never change
+        e(f"s_mov_b32 {s(S['RsrcX'] + 2)}, {self.sr('Slab')}")
+        e(f"s_mov_b32 {s(S['RsrcX'] + 3)}, 0x{FLAGS:x}")
+        e(f"s_mov_b32 {s(S['RsrcU'])}, {s(S['U'])}")
+        e(f"s_mov_b32 {s(S['RsrcU'] + 1)}, {s(S['U'] + 1)}")
+        e(f"s_mov_b32 {s(S['RsrcU'] + 2)}, {self.sr('UswBytes')}")
+        e(f"s_mov_b32 {s(S['RsrcU'] + 3)}, 0x{FLAGS:x}")
+        e(f"s_mov_b32 {s(S['RsrcY'] + 2)}, 0x{OOB:x}")
+        e(f"s_mov_b32 {s(S['RsrcY'] + 3)}, 0x{FLAGS:x}")
+        # per lane
+        tmp = lambda i: self.vr("Tmp", i)
+        e(f"v_lshrrev_b32 {tmp(0)}, 5, {self.vr('Lane')}")             # hsel
+        e(f"v_and_b32 {tmp(1)}, 31, {self.vr('Lane')}")                # nl
+        e(f"v_lshlrev_b32 {tmp(1)}, 2, {tmp(1)}")                      # nl*4
+        e(f"v_mul_lo_u32 {tmp(2)}, {tmp(0)}, {self.sr('HWN4')}")       # hsel*HWN*4
+        e(f"v_add_u32 {self.vr('LaneX')}, {tmp(2)}, {tmp(1)}")
+        e(f"v_lshlrev_b32 {tmp(2)}, 2, {tmp(2)}")                      # 4*hsel*HWN*4
+        e(f"v_add_u32 {self.vr('Off', 0)}, {tmp(2)}, {tmp(1)}")
+        e(f"v_add_u32 {self.vr('Off', 1)}, {self.sr('ColStep')}, {self.vr('Off', 0)}")
+        e(f"v_add_u32 {self.vr('Off', 2)}, {self.sr('RowStep')}, {self.vr('Off', 0)}")
+        e(f"v_add_u32 {self.vr('Off', 3)}, {self.sr('ColStep')}, {self.vr('Off', 2)}")
+        e(f"v_lshlrev_b32 {self.vr('Lane8')}, 3, {self.vr('Lane')}")
+        e(f"v_add_u32 {self.vr('Lane8b')}, 0x1000, {self.vr('Lane8')}")
+        # LDS: V[cw][buf][step][p][lane] floats.  Lds = read buffer, LdsWr = write buffer + this
+        # wave's first owned step; the prologue writes buffer 0, which the swap in end_of_chunk
+        # then makes the read buffer.
+        e(f"v_lshlrev_b32 {tmp(0)}, 2, {self.vr('Lane')}")
+        e(f"s_lshl_b32 {t(0)}, {self.sr('Cw')}, 15")
+        e(f"v_add_u32 {tmp(0)}, {t(0)}, {tmp(0)}")
+        e(f"v_add_u32 {self.vr('Lds')}, 0x4000, {tmp(0)}")
+        e(f"s_lshl_b32 {t(0)}, {self.sr('KwSpw')}, 12")
+        e(f"v_add_u32 {self.vr('LdsWr')}, {t(0)}, {tmp(0)}")
+
+        # ---- prologue: unit 0 -> buffer 0, patches of unit 1 and the first filter quad in flight
+        self.decode(self.sr("Tm"))
+        self.m_tile_setup()
+        e(f"s_mov_b32 {self.sr('KgQ')}, {self.sr('KgM')}")
+        self.patch_offsets()
+        self.u_offset(self.sr("UoffQ"), self.sr("KgM"), self.sr("Cm"), False)
+        for p in range(16):
+            self.load_u("U0", p, self.sr("UoffQ"))
+        for j in range(self.SPW):
+            self.slab_descriptor(j)
+            for p in range(16):
+                self.load_patch("D0" if j == 0 else "D1", p)
+        e("s_waitcnt vmcnt(0)")
+        for j in range(self.SPW):
+            self.transform("D0" if j == 0 else "D1", j)
+        e(f"s_mov_b32 {self.sr('G')}, -1")
+        self.advance_p()  # G + 2 = 1: on to unit 1 when there is one
+        for j in range(self.SPW):
+            self.slab_descriptor(j)
+            for p in range(16):
+                self.load_patch("D0" if j == 0 else "D1", p)
+        e(f"s_mov_b32 {self.sr('G')}, 0")
+        self.end_of_chunk()
+        e("s_waitcnt vmcnt(0)")
+
+        seg_loop, regular, check, done = (self.newlabel(x) for x in ("seg", "regular", "check", "done"))
+        plain_seg, epi_plain, after_epi = (self.newlabel(x) for x in ("plainseg", "epiplain", "afterepi"))
+        self.label(seg_loop)
+        # this segment: chunks Cm .. SegEnd-1 of tile Tm.  Kind: 1 publish (starts inside the tile),
+        # 2 merge (ends inside the tile), 0 whole tile.
+        e(f"s_sub_u32 {t(0)}, {self.sr('Nunits')}, {self.sr('G')}")
+        e(f"s_sub_u32 {t(1)}, {self.sr('Chunks')}, {self.sr('Cm')}")
+        e(f"s_min_u32 {t(0)}, {t(0)}, {t(1)}")
+        e(f"s_add_u32 {self.sr('SegEnd')}, {self.sr('Cm')}, {t(0)}")
+        e(f"s_cmp_lg_u32 {self.sr('Cm')}, 0")
+        e(f"s_cselect_b32 {self.sr('Kind')}, 1, 0")
+        e(f"s_cmp_lt_u32 {self.sr('SegEnd')}, {self.sr('Chunks')}")
+        e(f"s_cbranch_scc0 {plain_seg}")
+        e(f"s_mov_b32 {self.sr('Kind')}, 2")
+        self.merge_init()
+        e(f"s_branch {check}")
+        self.label(plain_seg)
+        self.chunk(True)
+        self.label(check)
+        e(f"s_cmp_lt_u32 {self.sr('Cm')}, {self.sr('SegEnd')}")
+        e(f"s_cbranch_scc0 {epi_plain}")
+        self.label(regular)
+        self.chunk(False)
+        e(f"s_cmp_lt_u32 {self.sr('Cm')}, {self.sr('SegEnd')}")
+        e(f"s_cbranch_scc1 {regular}")
+        self.label(epi_plain)
+        pub = self.newlabel("publish")
+        e(f"s_cmp_eq_u32 {self.sr('Kind')}, 1")
+        e(f"s_cbranch_scc1 {pub}")
+        self.epilogue(False)
+        e(f"s_branch {after_epi}")
+        self.label(pub)
+        self.epilogue(True)
+        e("s_waitcnt vmcnt(0)")  # every write-through store acknowledged, then the flag
+        self.flag_address(True)
+        self.store_flag(self.vr("One"))
+        e("s_waitcnt vmcnt(0)")
+        self.label(after_epi)
+        e(f"s_cmp_lt_u32 {self.sr('G')}, {self.sr('Nunits')}")
+        e(f"s_cbranch_scc0 {done}")
+        e(f"s_add_u32 {self.sr('Tm')}, {self.sr('Tm')}, 1")
+        e(f"s_mov_b32 {self.sr('Cm')}, 0")
+        self.decode(self.sr("Tm"))
+        self.m_tile_setup()
+        e(f"s_branch {seg_loop}")
+        self.label(done)
+        e("s_endpgm")
+
+    def emit(self, out):
+        self.body()
+        n = self.name
+        out.append(f"\t.text\n\t.protected\t{n}\n\t.globl\t{n}\n\t.p2align\t8\n\t.type\t{n},@function\n{n}:")
+        out.extend(self.lines)
+        out.append(f".L{n}_end:\n\t.size\t{n}, .L{n}_end-{n}")
+        out.append(f"""\t.rodata
+\t.p2align\t6
+\t.amdhsa_kernel {n}
+\t\t.amdhsa_group_segment_fixed_size 0
+\t\t.amdhsa_private_segment_fixed_size 0
+\t\t.amdhsa_kernarg_size 128
+\t\t.amdhsa_user_sgpr_count 2
+\t\t.amdhsa_user_sgpr_kernarg_segment_ptr 1
+\t\t.amdhsa_system_sgpr_workgroup_id_x 1
+\t\t.amdhsa_system_vgpr_workitem_id 0
+\t\t.amdhsa_next_free_vgpr 512
+\t\t.amdhsa_next_free_sgpr {self.sgpr_count}
+\t\t.amdhsa_accum_offset 256
+\t\t.amdhsa_reserve_vcc 1
+\t\t.amdhsa_float_round_mode_32 0
+\t\t.amdhsa_float_denorm_mode_32 3
+\t\t.amdhsa_float_denorm_mode_16_64 3
+\t\t.amdhsa_dx10_clamp 1
+\t\t.amdhsa_ieee_mode 1
+\t.end_amdhsa_kernel""")
+
+    def metadata(self):
+        args = "\n".join(f"""      - .address_space:  global
+        .offset:         {8 * i}
+        .size:           8
+        .value_kind:     global_buffer""" for i in range(4))
+        args += "\n" + "\n".join(f"""      - .offset:         {32 + 4 * i}
+        .size:           4
+        .value_kind:     by_value""" for i in range(24))
+        return f"""  - .agpr_count:     256
+    .args:
+{args}
+    .group_segment_fixed_size: 0
+    .kernarg_segment_align: 8
+    .kernarg_segment_size: 128
+    .max_flat_workgroup_size: 256
+    .name:           {self.name}
+    .private_segment_fixed_size: 0
+    .sgpr_count:     {self.sgpr_count + 6}
+    .sgpr_spill_count: 0
+    .symbol:         {self.name}.kd
+    .uniform_work_group_size: 1
+    .uses_dynamic_stack: false
+    .vgpr_count:     512
+    .vgpr_spill_count: 0
+    .wavefront_size: 64"""
+
+
+def main():
+    out = ['\t.amdgcn_target "amdgcn-amd-amdhsa--gfx950"', "\t.amdhsa_code_object_version 6"]
+    kernels = [Kernel(2), Kernel(4)]
+    for k in kernels:
+        k.emit(out)
+    out.append("\t.amdgpu_metadata\n---\namdhsa.kernels:")
+    out.extend(k.metadata() for k in kernels)
+    out.append("amdhsa.target:   amdgcn-amd-amdhsa--gfx950\namdhsa.version:\n  - 1\n  - 2\n...\n\t.end_amdgpu_metadata")
+    sys.stdout.write("\n".join(out) + "\n")
+
+
+if __name__ == "__main__":
+    main()

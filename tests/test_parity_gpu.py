@@ -243,26 +243,82 @@ def test_lds_variant_rejects_k_not_multiple_of_64(ocn, torch_gpu):
         ocn.set_kernel_variant(ocn.KERNEL_AUTO)
 
 
+@pytest.mark.parametrize("family", ["asm", "hip"])
 @pytest.mark.parametrize("N,C,H,K", [(64, 16, 40, 128), (32, 64, 45, 64), (96, 8, 33, 128)])
-def test_balanced_split_matches_plain_launch(ocn, oracle, torch_gpu, N, C, H, K):
+def test_balanced_split_matches_plain_launch(ocn, oracle, torch_gpu, N, C, H, K, family):
     # more workgroup tiles than CUs and not a whole number of rounds: the persistent,
     # evenly split launch merges tiles cut between two workgroups.  It must meet the bar,
-    # repeat bit for bit (the merge is a two-term sum), and stay within rounding of the
-    # plain one-tile-per-workgroup launch.
-    print(f"balanced N={N} C={C} H={H} K={K}", flush=True)
+    # repeat bit for bit (the merge does not depend on timing), and stay within rounding of the
+    # plain one-tile-per-workgroup launch.  Both kernel families implement it.
+    print(f"balanced {family} N={N} C={C} H={H} K={K}", flush=True)
     x, w = make_tensors(ocn, N, C, H, H, K)
     r = Runner(ocn, torch_gpu, x, w)
-    y1 = r.dropin()
-    y2 = r.dropin()
-    assert np.array_equal(y1, y2)
-    check_against_oracle(oracle, y1, x, w)
     try:
+        ocn.set_kernel_variant(ocn.KERNEL_ASM if family == "asm" else ocn.KERNEL_HIP)
+        y1 = r.dropin()
+        y2 = r.dropin()
+        ocn.set_kernel_variant(ocn.KERNEL_HIP)
         ocn.set_balanced_split(False)
         y0 = r.dropin()
     finally:
         ocn.set_balanced_split(True)
+        ocn.set_kernel_variant(ocn.KERNEL_AUTO)
+    assert np.array_equal(y1, y2)
+    check_against_oracle(oracle, y1, x, w)
     check_against_oracle(oracle, y0, x, w)
     np.testing.assert_allclose(y1, y0, rtol=0, atol=2e-6 * np.abs(y0).max())
+
+
+# (N, C, H, W, K): whole tiles per workgroup, tiles cut between workgroups, odd sizes, a missing
+# column tile in the last workgroup (odd number of column tiles), one and many chunks
+ASM_SHAPES = [(32, 8, 8, 8, 64), (64, 64, 8, 8, 64), (64, 16, 7, 15, 64), (32, 8, 7, 15, 256),
+              (64, 32, 16, 16, 128), (64, 24, 31, 31, 64), (32, 40, 45, 45, 64), (32, 16, 63, 5, 128)]
+
+
+@pytest.mark.parametrize("N,C,H,W,K", ASM_SHAPES)
+def test_assembly_kernels(ocn, oracle, torch_gpu, N, C, H, W, K):
+    # the hand-scheduled kernels selected explicitly (an unsupported shape would raise, not fall
+    # back), against the fp64 direct convolution and bit for bit against a second call
+    print(f"asm N={N} C={C} H={H} W={W} K={K}", flush=True)
+    x, w = make_tensors(ocn, N, C, H, W, K)
+    r = Runner(ocn, torch_gpu, x, w)
+    try:
+        ocn.set_kernel_variant(ocn.KERNEL_ASM)
+        y = r.split()
+        y2 = r.split()
+    finally:
+        ocn.set_kernel_variant(ocn.KERNEL_AUTO)
+    assert not np.isnan(y).any(), "an output element was never written"
+    assert np.array_equal(y, y2)
+    rel64, _, _ = oracle.compare(y, oracle.direct_conv_f64(x, w))
+    assert rel64 <= 1e-5, f"rel-L2 vs fp64 direct {rel64:.3e}"
+    if H == W:
+        check_against_oracle(oracle, y, x, w)
+
+
+@pytest.mark.parametrize("name,N,C,H,K,xr,filt", CONFIGS[1:], ids=[c[0] for c in CONFIGS[1:]])
+def test_benchmark_configs_on_hip_kernels(ocn, oracle, torch_gpu, name, N, C, H, K, xr, filt):
+    # test_benchmark_configs runs the default choice (the assembly kernels on these layers); the
+    # HIP C++ kernels stay the path for every shape the assembly does not take
+    print(f"hip config {name}", flush=True)
+    x, w = make_tensors(ocn, N, C, H, H, K, xr, filt)
+    try:
+        ocn.set_kernel_variant(ocn.KERNEL_HIP)
+        y = Runner(ocn, torch_gpu, x, w).dropin()
+    finally:
+        ocn.set_kernel_variant(ocn.KERNEL_AUTO)
+    check_against_oracle(oracle, y, x, w)
+
+
+def test_assembly_variant_rejects_shapes_it_does_not_take(ocn, torch_gpu):
+    x, w = make_tensors(ocn, 32, 8, 6, 6, 96)  # three filter groups: no whole filter block
+    r = Runner(ocn, torch_gpu, x, w)
+    try:
+        ocn.set_kernel_variant(ocn.KERNEL_ASM)
+        with pytest.raises(ocn.OpenCNNError):
+            r.dropin()
+    finally:
+        ocn.set_kernel_variant(ocn.KERNEL_AUTO)
 
 
 # ---------------------------------------------------------------- shapes outside the reference's tiling
