@@ -62,6 +62,7 @@ class Kernel:
         self.CW = 4 // KW
         self.SPW = 4 // KW
         self.lines = []
+        self.outofline = []  # rarely executed blocks, emitted behind s_endpgm
         self.nlabel = 0
         self.name = f"wino_f32_asm_kw{KW}"
         self.alloc()
@@ -275,9 +276,10 @@ class Kernel:
         for p in range(0, 16, 2):
             self.e(f"ds_write2st64_b32 {self.vr('LdsWr')}, {o(p)}, {o(p + 1)} offset0:{j * 16 + p} offset1:{j * 16 + p + 1}")
 
-    def mfma_step(self, step, first, vmem):
+    def mfma_step(self, step, first, vmem, scalar_work=None):
         """16 MFMAs of one step; behind MFMA p: vmem(p) (one global load or nothing) and, for
-        p < 8, the LDS read of two B operands of the next step."""
+        p < 8, the LDS read of two B operands of the next step.  scalar_work() is emitted behind
+        the first MFMA: scalar instructions issue while the matrix pipe is busy."""
         usrc = "U0" if step < 2 else "U1"
         vsrc = "VA" if step % 2 == 0 else "VB"
         vnext = "VB" if step % 2 == 0 else "VA"
@@ -288,6 +290,8 @@ class Kernel:
                 vmem(p)
             if step < 3 and p < 8:
                 self.read_v(vnext, step + 1, 2 * p)
+            if p == 0 and scalar_work:
+                scalar_work()
 
     def end_of_chunk(self):
         """All LDS traffic of this wave done, workgroup barrier, swap the buffers, fetch the first
@@ -301,35 +305,45 @@ class Kernel:
 
     # ------------------------------------------------------------------ cursors
     def advance_p(self):
-        skip = self.newlabel("skip_p")
+        """P cursor -> unit G+2 when there is one.  The common case (same tile) falls through
+        without a taken branch; the tile switch lives out of line, behind the kernel's end."""
+        rare, back = self.newlabel("p_switch"), self.newlabel("p_back")
         t = self.t
         self.e(f"s_add_u32 {t(0)}, {self.sr('G')}, 2")
         self.e(f"s_cmp_lt_u32 {t(0)}, {self.sr('Nunits')}")
-        self.e(f"s_cbranch_scc0 {skip}")
-        self.e(f"s_add_u32 {self.sr('Cp')}, {self.sr('Cp')}, 1")
-        self.e(f"s_cmp_lt_u32 {self.sr('Cp')}, {self.sr('Chunks')}")
-        self.e(f"s_cbranch_scc1 {skip}")
+        self.e(f"s_addc_u32 {self.sr('Cp')}, {self.sr('Cp')}, 0")  # + SCC
+        self.e(f"s_cmp_eq_u32 {self.sr('Cp')}, {self.sr('Chunks')}")
+        self.e(f"s_cbranch_scc1 {rare}")
+        self.label(back)
+        main, self.lines = self.lines, []
+        self.label(rare)
         self.e(f"s_mov_b32 {self.sr('Cp')}, 0")
         self.e(f"s_add_u32 {self.sr('Tp')}, {self.sr('Tp')}, 1")
         self.decode(self.sr("Tp"))
         self.patch_offsets()
-        self.label(skip)
+        self.e(f"s_branch {back}")
+        self.outofline.extend(self.lines)
+        self.lines = main
 
     def advance_q(self):
-        skip = self.newlabel("skip_q")
+        rare, back = self.newlabel("q_switch"), self.newlabel("q_back")
         t = self.t
         self.e(f"s_add_u32 {t(0)}, {self.sr('G')}, 1")
         self.e(f"s_cmp_lt_u32 {t(0)}, {self.sr('Nunits')}")
-        self.e(f"s_cbranch_scc0 {skip}")
-        self.e(f"s_add_u32 {self.sr('Cq')}, {self.sr('Cq')}, 1")
-        self.e(f"s_cmp_lt_u32 {self.sr('Cq')}, {self.sr('Chunks')}")
-        self.e(f"s_cbranch_scc1 {skip}")
+        self.e(f"s_addc_u32 {self.sr('Cq')}, {self.sr('Cq')}, 0")
+        self.e(f"s_cmp_eq_u32 {self.sr('Cq')}, {self.sr('Chunks')}")
+        self.e(f"s_cbranch_scc1 {rare}")
+        self.label(back)
+        main, self.lines = self.lines, []
+        self.label(rare)
         self.e(f"s_mov_b32 {self.sr('Cq')}, 0")
         self.e(f"s_add_u32 {self.sr('Tq')}, {self.sr('Tq')}, 1")
         self.div(t(0), self.sr("Tq"), self.sr("Mcb"), self.sr("Scb"))
         self.e(f"s_lshl_b32 {t(0)}, {t(0)}, {self.KW.bit_length() - 1}")
         self.e(f"s_add_u32 {self.sr('KgQ')}, {t(0)}, {self.sr('Kw')}")
-        self.label(skip)
+        self.e(f"s_branch {back}")
+        self.outofline.extend(self.lines)
+        self.lines = main
 
     # ------------------------------------------------------------------ one chunk
     def chunk(self, first):
@@ -343,15 +357,18 @@ class Kernel:
         two = self.SPW == 2
         wait = lambda n: self.e(f"s_waitcnt vmcnt({min(63, n + (64 if first else 0))})")
         self.comment(f"---- chunk ({'first of a segment' if first else 'steady state'})")
-        self.advance_p()
-        self.advance_q()
         # step 0
         wait(32 if two else 16)  # D0 of unit G+1 has landed
         self.transform("D0", 0)
         self.u_offset(self.sr("UoffM"), self.sr("KgM"), self.sr("Cm"), True)
         wait(16 if two else 0)  # U0 of this unit has landed
         self.e("s_waitcnt lgkmcnt(8)")  # first B operands (the 8 LDS writes above may still fly)
-        self.mfma_step(0, first, lambda p: self.load_u("U1", p, self.sr("UoffM")))
+        # The cursors move behind the first MFMA (the patch loads of step 1 and the filter loads
+        # of step 2 are their first users); in front of the chunk the matrix pipe would wait.
+        def cursors():
+            self.advance_p()
+            self.advance_q()
+        self.mfma_step(0, first, lambda p: self.load_u("U1", p, self.sr("UoffM")), cursors)
         # step 1
         self.slab_descriptor(0)
         self.e("s_waitcnt lgkmcnt(0)")
@@ -630,6 +647,7 @@ class Kernel:
         e(f"s_branch {seg_loop}")
         self.label(done)
         e("s_endpgm")
+        self.lines.extend(self.outofline)
 
     def emit(self, out):
         self.body()
