@@ -257,9 +257,9 @@ class Kernel:
         """Two B operands (positions p, p+1) of MFMA step `step` from the read buffer."""
         self.e(f"ds_read2st64_b32 {self.vr(dst, p, 2)}, {self.vr('Lds')} offset0:{step * 16 + p} offset1:{step * 16 + p + 1}")
 
-    def transform(self, src, j):
+    def transform(self, src):
         """V = B^T d B of one patch (columns first, then rows, the order of
-        src/convolutionForward_32x64x8.cu:59-80), written to the write buffer as owned step j."""
+        src/convolutionForward_32x64x8.cu:59-80), left in TO[0..15] for write_v."""
         d = lambda i: self.vr(src, i)
         t = lambda i: self.vr("T", i)
         o = lambda i: self.vr("TO", i)
@@ -273,13 +273,18 @@ class Kernel:
             self.e(f"v_add_f32 {o(4 * r + 1)}, {t(4 * r + 1)}, {t(4 * r + 2)}")
             self.e(f"v_sub_f32 {o(4 * r + 2)}, {t(4 * r + 2)}, {t(4 * r + 1)}")
             self.e(f"v_sub_f32 {o(4 * r + 3)}, {t(4 * r + 1)}, {t(4 * r + 3)}")
-        for p in range(0, 16, 2):
-            self.e(f"ds_write2st64_b32 {self.vr('LdsWr')}, {o(p)}, {o(p + 1)} offset0:{j * 16 + p} offset1:{j * 16 + p + 1}")
 
-    def mfma_step(self, step, first, vmem, scalar_work=None):
+    def write_v(self, j, p):
+        """Two transformed values (positions p, p+1) of owned step j to the write buffer."""
+        o = lambda i: self.vr("TO", i)
+        self.e(f"ds_write2st64_b32 {self.vr('LdsWr')}, {o(p)}, {o(p + 1)} offset0:{j * 16 + p} offset1:{j * 16 + p + 1}")
+
+    def mfma_step(self, step, first, vmem, scalar_work=None, write_step=None):
         """16 MFMAs of one step; behind MFMA p: vmem(p) (one global load or nothing) and, for
         p < 8, the LDS read of two B operands of the next step.  scalar_work() is emitted behind
-        the first MFMA: scalar instructions issue while the matrix pipe is busy."""
+        the first MFMA: scalar instructions issue while the matrix pipe is busy.  write_step: the
+        transformed patch waiting in TO goes to LDS as owned step `write_step`, two values
+        behind each of the first eight MFMAs."""
         usrc = "U0" if step < 2 else "U1"
         vsrc = "VA" if step % 2 == 0 else "VB"
         vnext = "VB" if step % 2 == 0 else "VA"
@@ -290,6 +295,8 @@ class Kernel:
                 vmem(p)
             if step < 3 and p < 8:
                 self.read_v(vnext, step + 1, 2 * p)
+            if write_step is not None and p < 8:
+                self.write_v(write_step, 2 * p)
             if p == 0 and scalar_work:
                 scalar_work()
 
@@ -359,16 +366,16 @@ class Kernel:
         self.comment(f"---- chunk ({'first of a segment' if first else 'steady state'})")
         # step 0
         wait(32 if two else 16)  # D0 of unit G+1 has landed
-        self.transform("D0", 0)
+        self.transform("D0")
         self.u_offset(self.sr("UoffM"), self.sr("KgM"), self.sr("Cm"), True)
         wait(16 if two else 0)  # U0 of this unit has landed
-        self.e("s_waitcnt lgkmcnt(8)")  # first B operands (the 8 LDS writes above may still fly)
+        self.e("s_waitcnt lgkmcnt(0)")  # first B operands
         # The cursors move behind the first MFMA (the patch loads of step 1 and the filter loads
         # of step 2 are their first users); in front of the chunk the matrix pipe would wait.
         def cursors():
             self.advance_p()
             self.advance_q()
-        self.mfma_step(0, first, lambda p: self.load_u("U1", p, self.sr("UoffM")), cursors)
+        self.mfma_step(0, first, lambda p: self.load_u("U1", p, self.sr("UoffM")), cursors, write_step=0)
         # step 1
         self.slab_descriptor(0)
         self.e("s_waitcnt lgkmcnt(0)")
@@ -376,11 +383,11 @@ class Kernel:
         # step 2
         if two:
             self.e("s_waitcnt vmcnt(%d)" % (63 if first else 32))  # D1 of unit G+1 has landed
-            self.transform("D1", 1)
+            self.transform("D1")
         self.u_offset(self.sr("UoffQ"), self.sr("KgQ"), self.sr("Cq"), False)
         self.e("s_waitcnt vmcnt(16)")  # U1 (step 0) has landed; only D0 (step 1) is younger
-        self.e("s_waitcnt lgkmcnt(%d)" % (8 if two else 0))
-        self.mfma_step(2, first, lambda p: self.load_u("U0", p, self.sr("UoffQ")))
+        self.e("s_waitcnt lgkmcnt(0)")
+        self.mfma_step(2, first, lambda p: self.load_u("U0", p, self.sr("UoffQ")), write_step=1 if two else None)
         # step 3
         if two:
             self.slab_descriptor(1)
@@ -413,11 +420,16 @@ class Kernel:
         self.e("s_nop 15")
         self.e("s_nop 15")
         m = lambda i: self.vr("T", i)
+        pending = []
         for r in range(16):
             w = lambda i: self.vr("TO", i)          # a_j: 0-3, b_j: 4-7
             o = lambda q: self.vr("TO", 8 + 4 * (r & 1) + q)  # outputs alternate between two sets
             for p in range(16):
                 self.e(f"v_accvgpr_read_b32 {m(p)}, {a(16 * p + r)}")
+            if r > 0:  # the previous row's outputs, now certainly computed: store, then move on a row
+                for st in pending:
+                    self.e(st)
+                self.row_advance(r - 1)
             for j in range(4):
                 self.e(f"v_add_f32 {w(j)}, {m(j)}, {m(4 + j)}")
                 self.e(f"v_sub_f32 {w(4 + j)}, {m(4 + j)}, {m(8 + j)}")
@@ -432,9 +444,10 @@ class Kernel:
             self.e(f"v_sub_f32 {o(1)}, {o(1)}, {w(3)}")
             self.e(f"v_add_f32 {o(2)}, {o(2)}, {w(6)}")
             self.e(f"v_sub_f32 {o(3)}, {o(3)}, {w(7)}")
-            for q in range(4):
-                self.e(f"buffer_store_dword {o(q)}, {self.vr('Eff', q)}, {s(ry, 4)}, 0 offen{pol}")
-            self.row_advance(r)
+            pending = [f"buffer_store_dword {o(q)}, {self.vr('Eff', q)}, {s(ry, 4)}, 0 offen{pol}" for q in range(4)]
+            if r == 15:
+                for st in pending:
+                    self.e(st)
 
     def flag_address(self, previous):
         """Fl = &flags[((L - previous) * 4 + wave) * 2 + 1]."""
@@ -589,7 +602,9 @@ class Kernel:
                 self.load_patch("D0" if j == 0 else "D1", p)
         e("s_waitcnt vmcnt(0)")
         for j in range(self.SPW):
-            self.transform("D0" if j == 0 else "D1", j)
+            self.transform("D0" if j == 0 else "D1")
+            for p in range(0, 16, 2):
+                self.write_v(j, p)
         e(f"s_mov_b32 {self.sr('G')}, -1")
         self.advance_p()  # G + 2 = 1: on to unit 1 when there is one
         for j in range(self.SPW):
