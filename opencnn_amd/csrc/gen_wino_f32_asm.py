@@ -588,23 +588,21 @@ class Kernel:
         e(f"s_lshl_b32 {t(0)}, {self.sr('KwSpw')}, 12")
         e(f"v_add_u32 {self.vr('LdsWr')}, {t(0)}, {tmp(0)}")
 
-        # ---- prologue: unit 0 -> buffer 0, patches of unit 1 and the first filter quad in flight
+        # ---- prologue: unit 0 -> buffer 0 with the patches of unit 1 already in flight.  Unit 0's
+        # patches land in registers that are free until the first chunk (MPX, VB), so that both
+        # units' loads leave together and the kernel pays one trip to memory, not two.
         self.decode(self.sr("Tm"))
         self.m_tile_setup()
         e(f"s_mov_b32 {self.sr('KgQ')}, {self.sr('KgM')}")
         self.patch_offsets()
         self.u_offset(self.sr("UoffQ"), self.sr("KgM"), self.sr("Cm"), False)
-        for p in range(16):
-            self.load_u("U0", p, self.sr("UoffQ"))
+        first_patch = ["MPX", "VB"]
         for j in range(self.SPW):
             self.slab_descriptor(j)
             for p in range(16):
-                self.load_patch("D0" if j == 0 else "D1", p)
-        e("s_waitcnt vmcnt(0)")
-        for j in range(self.SPW):
-            self.transform("D0" if j == 0 else "D1")
-            for p in range(0, 16, 2):
-                self.write_v(j, p)
+                self.load_patch(first_patch[j], p)
+        for p in range(16):
+            self.load_u("U0", p, self.sr("UoffQ"))
         e(f"s_mov_b32 {self.sr('G')}, -1")
         self.advance_p()  # G + 2 = 1: on to unit 1 when there is one
         for j in range(self.SPW):
@@ -612,8 +610,13 @@ class Kernel:
             for p in range(16):
                 self.load_patch("D0" if j == 0 else "D1", p)
         e(f"s_mov_b32 {self.sr('G')}, 0")
+        e(f"s_waitcnt vmcnt({16 * self.SPW})")  # everything but unit 1's patches
+        for j in range(self.SPW):
+            self.transform(first_patch[j])
+            for p in range(0, 16, 2):
+                self.write_v(j, p)
         self.end_of_chunk()
-        e("s_waitcnt vmcnt(0)")
+        e("s_waitcnt vmcnt(0)")  # the first chunk counts on a queue without surprises
 
         seg_loop, regular, check, done = (self.newlabel(x) for x in ("seg", "regular", "check", "done"))
         plain_seg, epi_plain, after_epi = (self.newlabel(x) for x in ("plainseg", "epiplain", "afterepi"))
