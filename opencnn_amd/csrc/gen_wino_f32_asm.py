@@ -29,6 +29,9 @@ import sys
 
 OOB = 0x80000000
 FLAGS = 0x00020000
+# A^T M A is linear: output (a,b) of a 2x2 tile is the image of Winograd position (0,0), -(0,3),
+# -(3,0), (3,3).  position -> (output index, negate)
+MERGE_POSITIONS = {0: (0, False), 3: (1, True), 12: (2, True), 15: (3, False)}
 
 
 class Alloc:
@@ -289,7 +292,8 @@ class Kernel:
         vsrc = "VA" if step % 2 == 0 else "VB"
         vnext = "VB" if step % 2 == 0 else "VA"
         for p in range(16):
-            c = "0" if (first and step == 0) else a(16 * p, 16)
+            fresh = first and step == 0 and not (first == "merge" and p in MERGE_POSITIONS)
+            c = "0" if fresh else a(16 * p, 16)
             self.e(f"v_mfma_f32_32x32x2_f32 {a(16 * p, 16)}, {self.vr(usrc, 2 * p + (step & 1))}, {self.vr(vsrc, p)}, {c}")
             if vmem:
                 vmem(p)
@@ -363,7 +367,7 @@ class Kernel:
         for is older than those stores and the counts grow by 64 (capped at the field's 63)."""
         two = self.SPW == 2
         wait = lambda n: self.e(f"s_waitcnt vmcnt({min(63, n + (64 if first else 0))})")
-        self.comment(f"---- chunk ({'first of a segment' if first else 'steady state'})")
+        self.comment(f"---- chunk ({'first of a segment (' + str(first) + ')' if first else 'steady state'})")
         # step 0
         wait(32 if two else 16)  # D0 of unit G+1 has landed
         self.transform("D0")
@@ -496,18 +500,14 @@ class Kernel:
                 self.e(f"buffer_load_dword {v(self.MP[r * 4 + q])}, {self.vr('Eff', q)}, {s(ry, 4)}, 0 offen sc0 sc1")
             self.row_advance(r)
         self.e("s_waitcnt vmcnt(0)")
-        # outputs (a,b) of a 2x2 tile <- positions (0,0), -(0,3), -(3,0), (3,3)
-        src = {0: (0, False), 3: (1, True), 12: (2, True), 15: (3, False)}
-        for p in range(16):
+        # the four positions that carry the partial outputs; the other twelve start from the
+        # constant 0 in the first MFMA step of the segment
+        for p, (q, neg) in MERGE_POSITIONS.items():
             for r in range(16):
-                if p in src:
-                    q, neg = src[p]
-                    reg = v(self.MP[r * 4 + q])
-                    if neg:
-                        self.e(f"v_xor_b32 {reg}, 0x80000000, {reg}")
-                    self.e(f"v_accvgpr_write_b32 {a(16 * p + r)}, {reg}")
-                else:
-                    self.e(f"v_accvgpr_write_b32 {a(16 * p + r)}, 0")
+                reg = v(self.MP[r * 4 + q])
+                if neg:
+                    self.e(f"v_xor_b32 {reg}, 0x80000000, {reg}")
+                self.e(f"v_accvgpr_write_b32 {a(16 * p + r)}, {reg}")
         self.store_flag(self.vr("Zero"))  # hand the flag back for the next launch
         self.e("s_nop 15")
         self.e("s_nop 15")
@@ -633,6 +633,7 @@ class Kernel:
         e(f"s_cbranch_scc0 {plain_seg}")
         e(f"s_mov_b32 {self.sr('Kind')}, 2")
         self.merge_init()
+        self.chunk("merge")
         e(f"s_branch {check}")
         self.label(plain_seg)
         self.chunk(True)
