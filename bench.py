@@ -41,10 +41,10 @@ DEFAULT_WORKLOAD = "resnet_n64_c64_h56_k64"
 # HBM bytes per launch of the fused kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # (profiles/), or None where not measured yet.
 MEASURED_TRAFFIC_BYTES = {
-    "resnet_n64_c64_h56_k64": 265.1e6,
-    "resnet_n128_c128_h28_k128": 267.0e6,
-    "deep_n128_c256_h14_k256": 255.4e6,
-    "deep_n128_c512_h7_k512": 116.7e6,
+    "resnet_n64_c64_h56_k64": 215.6e6,
+    "resnet_n128_c128_h28_k128": 261.3e6,
+    "deep_n128_c256_h14_k256": 250.1e6,
+    "deep_n128_c512_h7_k512": 112.7e6,
 }
 
 
@@ -189,7 +189,7 @@ def main():
                    "W": layer.H, "K": layer.K, "pad": 1, "stride": 1,
                    "layout": "CHWN in, CRSK filters, KHWN out"},
         "roofline": {
-            "kernel": "wino_f32_stream / wino_f32_fused_lds (fused Winograd kernel)",
+            "kernel": "wino_f32_asm_kw2 / wino_f32_asm_kw4 (fused Winograd kernel, hand-scheduled assembly)",
             "bound": "mfma",
             "achieved": achieved,
             "peak": PEAK_FP32_MFMA_TFLOPS,
