@@ -256,8 +256,8 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   dim3 grid(per_xcd * 8), block(256);
   const size_t lds_bytes = (size_t)cw * 2 * 4 * 16 * 64 * sizeof(float);
   // Hand-scheduled kernels: one persistent launch whose workgroups share the (tile, chunk) units
-  // evenly.  They need whole filter blocks, a grid that divides into the 8 XCDs and at least one
-  // tile per workgroup (a tile then has at most two contributors).
+  // evenly.  They need whole filter blocks and at least one tile per workgroup (a tile then has
+  // at most two contributors).
   int agrid = 0;
   if ((variant == OPENCNN_KERNEL_ASM || variant == OPENCNN_KERNEL_AUTO) && !ragged && kw > 1 &&
       (long long)a.nblocks * (in_c / 8) <= kMaxElems &&
@@ -269,8 +269,8 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
       if (cus_asm % 8 == 0 && cus_asm <= opencnn::kMaxBalancedBlocks &&
           (a.nblocks % cus_asm == 0 || g_balance.load() != 0))
         agrid = cus_asm;
-    } else if (a.nblocks % 8 == 0) {
-      agrid = a.nblocks;
+    } else {
+      agrid = a.nblocks;  // one tile per workgroup
     }
   }
   if (variant == OPENCNN_KERNEL_ASM) REQUIRE(agrid > 0);
@@ -297,7 +297,7 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
     ka.units_q = (int32_t)(total / agrid);
     ka.units_rem = (int32_t)(total % agrid);
     ka.usw_bytes = (int32_t)((long long)in_c * 16 * filt_k * 4);
-    ka.grid_per_xcd = agrid / 8;
+    ka.grid_per_xcd = agrid % 8 == 0 ? agrid / 8 : 0;  // 0: no XCD-aware block order
     magic_divisor((uint32_t)chunks, &ka.m_chunks, &ka.s_chunks);
     magic_divisor((uint32_t)a.colblocks, &ka.m_colblocks, &ka.s_colblocks);
     magic_divisor((uint32_t)a.ngroups, &ka.m_ngroups, &ka.s_ngroups);

@@ -534,10 +534,13 @@ class Kernel:
         e(f"s_lshr_b32 {self.sr('Cw')}, {self.sr('Wave')}, {KWLOG}")
         e(f"s_mul_i32 {self.sr('KwSpw')}, {self.sr('Kw')}, {self.SPW}")
         # logical block: workgroups are dealt round-robin to the 8 XCDs; each XCD gets a contiguous range
+        # (GridPerXcd == 0: a grid that does not divide by 8, a small layer; blocks in launch order)
         e(f"s_and_b32 {t(0)}, s2, 7")
         e(f"s_mul_i32 {t(0)}, {t(0)}, {self.sr('GridPerXcd')}")
         e(f"s_lshr_b32 {t(1)}, s2, 3")
-        e(f"s_add_u32 {self.sr('L')}, {t(0)}, {t(1)}")
+        e(f"s_add_u32 {t(0)}, {t(0)}, {t(1)}")
+        e(f"s_cmp_eq_u32 {self.sr('GridPerXcd')}, 0")
+        e(f"s_cselect_b32 {self.sr('L')}, s2, {t(0)}")
         # units [Begin, Begin + Nunits): the first UnitsRem blocks take one more
         e(f"s_mul_i32 {self.sr('Begin')}, {self.sr('L')}, {self.sr('UnitsQ')}")
         e(f"s_min_u32 {t(0)}, {self.sr('L')}, {self.sr('UnitsRem')}")

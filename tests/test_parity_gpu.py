@@ -272,7 +272,9 @@ def test_balanced_split_matches_plain_launch(ocn, oracle, torch_gpu, N, C, H, K,
 # (N, C, H, W, K): whole tiles per workgroup, tiles cut between workgroups, odd sizes, a missing
 # column tile in the last workgroup (odd number of column tiles), one and many chunks
 ASM_SHAPES = [(32, 8, 8, 8, 64), (64, 64, 8, 8, 64), (64, 16, 7, 15, 64), (32, 8, 7, 15, 256),
-              (64, 32, 16, 16, 128), (64, 24, 31, 31, 64), (32, 40, 45, 45, 64), (32, 16, 63, 5, 128)]
+              (64, 32, 16, 16, 128), (64, 24, 31, 31, 64), (32, 40, 45, 45, 64), (32, 16, 63, 5, 128),
+              (32, 8, 1, 1, 64), (32, 16, 3, 5, 128), (96, 40, 21, 27, 64), (32, 8, 112, 112, 64),
+              (32, 1024, 7, 7, 1024), (256, 64, 28, 28, 64)]
 
 
 @pytest.mark.parametrize("N,C,H,W,K", ASM_SHAPES)
