@@ -1,0 +1,73 @@
+"""CPU checks of the assembly generator (opencnn_amd/csrc/gen_wino_f32_asm.py): it runs, stays
+inside the register file, keeps the invariants its wait counts rely on, and its output assembles
+for gfx950 (no GPU needed: the assembler cross-compiles)."""
+import importlib.util
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GEN = os.path.join(ROOT, "opencnn_amd", "csrc", "gen_wino_f32_asm.py")
+CLANG = "/opt/rocm/lib/llvm/bin/clang"
+
+
+@pytest.fixture(scope="module")
+def gen():
+    spec = importlib.util.spec_from_file_location("gen_wino_f32_asm", GEN)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+@pytest.mark.parametrize("kw", [2, 4])
+def test_register_budget(gen, kw):
+    k = gen.Kernel(kw)
+    assert k.vgpr_count <= 256          # arch VGPRs; the 256 accumulators are AGPRs
+    assert k.sgpr_count <= 96           # + VCC and the reserved registers of the target = 102
+    assert len(set(k.MP)) == 64         # landing registers of a published partial tile
+    live_at_boundary = set()
+    for name in ("U0", "U1", "D0", "D1", "VA", "VOFF", "Off", "Eff"):
+        if name in k.V:
+            n = {"U0": 32, "U1": 32, "D0": 16, "D1": 16, "VA": 16, "VOFF": 16, "Off": 4, "Eff": 4}[name]
+            live_at_boundary |= set(range(k.V[name], k.V[name] + n))
+    assert not live_at_boundary & set(k.MP), "partial tile would land on live pipeline registers"
+
+
+@pytest.mark.parametrize("kw", [2, 4])
+def test_kernel_text_invariants(gen, kw):
+    k = gen.Kernel(kw)
+    k.body()
+    text = "\n".join(k.lines)
+    # one workgroup barrier per chunk variant + the prologue; three chunk variants
+    assert text.count("s_barrier") == 4
+    # 64 MFMAs per chunk variant
+    assert len(re.findall(r"v_mfma_f32_32x32x2_f32", text)) == 3 * 64
+    # first step of a tile: 16 MFMAs from the constant 0; a merging segment keeps four accumulators
+    assert len(re.findall(r"v_mfma_f32_32x32x2_f32 [^\n]*, 0$", text, re.M)) == 16 + 12
+    # the counted waits rely on exactly 64 stores per epilogue (two epilogues: plain, publishing)
+    assert len(re.findall(r"buffer_store_dword", text)) == 2 * 64
+    assert len(re.findall(r"buffer_store_dword [^\n]* sc0 sc1", text)) == 64
+    # s_waitcnt fields: vmcnt has 6 bits, lgkmcnt 4
+    assert all(int(n) <= 63 for n in re.findall(r"vmcnt\((\d+)\)", text))
+    assert all(int(n) <= 15 for n in re.findall(r"lgkmcnt\((\d+)\)", text))
+    # every label that is branched to exists exactly once
+    labels = re.findall(r"^(\.L\w+):", text, re.M)
+    assert len(labels) == len(set(labels))
+    for target in re.findall(r"s_c?branch\w* (\.L\w+)", text):
+        assert target in labels
+
+
+@pytest.mark.skipif(not os.path.exists(CLANG), reason="ROCm LLVM assembler not installed")
+def test_output_assembles_for_gfx950(tmp_path):
+    src = tmp_path / "k.s"
+    with open(src, "w") as f:
+        subprocess.run(["python3", GEN], check=True, stdout=f)
+    obj = tmp_path / "k.o"
+    subprocess.run([CLANG, "-x", "assembler", "-target", "amdgcn-amd-amdhsa", "-mcpu=gfx950",
+                    "-c", str(src), "-o", str(obj)], check=True)
+    assert obj.stat().st_size > 10000
+    lld = shutil.which("ld.lld") or "/opt/rocm/lib/llvm/bin/ld.lld"
+    subprocess.run([lld, "-shared", str(obj), "-o", str(tmp_path / "k.hsaco")], check=True)
