@@ -128,10 +128,10 @@ int opencnn_set_stream(void *stream);
  *                            filter groups, otherwise later launches return
  *                            hipErrorInvalidValue)
  *   OPENCNN_KERNEL_ASM       the LDS scheme as hand-scheduled gfx950 assembly, one persistent
- *                            launch over all (tile, 8-channel chunk) units.  Needs in_n % 32 == 0,
- *                            in_c % 8 == 0, filt_k % 64 == 0 (and, for more workgroup tiles than
- *                            compute units that are not a multiple of them, the balanced split
- *                            switched on); otherwise later launches return hipErrorInvalidValue
+ *                            launch over all (tile, 8-channel chunk) units.  Needs an even number
+ *                            of 32-wide filter groups (and, for more workgroup tiles than compute
+ *                            units that are not a multiple of them, the balanced split switched
+ *                            on); otherwise later launches return hipErrorInvalidValue
  *   OPENCNN_KERNEL_HIP       the HIP C++ kernels only: the LDS variant when the 32-wide filter
  *                            groups (filt_k / 32, rounded up) pair up (as one continuous pipeline
  *                            over all tiles of a workgroup when the balanced split is in use),

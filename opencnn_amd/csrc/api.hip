@@ -45,7 +45,7 @@ extern "C" const char opencnn_wino_f32_asm_hsaco[];
 
 struct AsmKernels {
   hipModule_t module = nullptr;
-  hipFunction_t kw2 = nullptr, kw4 = nullptr;
+  hipFunction_t kw2 = nullptr, kw4 = nullptr, kw2_ragged = nullptr, kw4_ragged = nullptr;
   unsigned* split_sync = nullptr;  // device address of g_split_sync on this device
   bool ready = false;
 };
@@ -64,6 +64,8 @@ int asm_kernels(const AsmKernels** out) {
     if ((e = hipModuleLoadData(&k.module, opencnn_wino_f32_asm_hsaco)) != hipSuccess) return (int)e;
     if ((e = hipModuleGetFunction(&k.kw2, k.module, "wino_f32_asm_kw2")) != hipSuccess) return (int)e;
     if ((e = hipModuleGetFunction(&k.kw4, k.module, "wino_f32_asm_kw4")) != hipSuccess) return (int)e;
+    if ((e = hipModuleGetFunction(&k.kw2_ragged, k.module, "wino_f32_asm_kw2_ragged")) != hipSuccess) return (int)e;
+    if ((e = hipModuleGetFunction(&k.kw4_ragged, k.module, "wino_f32_asm_kw4_ragged")) != hipSuccess) return (int)e;
     if ((e = hipGetSymbolAddress(reinterpret_cast<void**>(&k.split_sync), HIP_SYMBOL(opencnn::g_split_sync))) != hipSuccess)
       return (int)e;
     // 64 KB of dynamic LDS for KW = 2 is the default limit exactly; nothing to raise
@@ -82,7 +84,7 @@ struct AsmKernArgs {
   int32_t N, H, W, chunks, tiles_w, ngroups, colgroups, colblocks;
   int32_t Q, HWN4, units_q, units_rem, usw_bytes, grid_per_xcd;
   uint32_t m_chunks, s_chunks, m_colblocks, s_colblocks, m_ngroups, s_ngroups, m_tiles_w, s_tiles_w;
-  int32_t spare[2];
+  int32_t c_real, k_real;  // read by the _ragged kernels only
 };
 static_assert(sizeof(AsmKernArgs) == 128, "kernel argument block");
 
@@ -259,8 +261,9 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   // evenly.  They need whole filter blocks and at least one tile per workgroup (a tile then has
   // at most two contributors).
   int agrid = 0;
-  if ((variant == OPENCNN_KERNEL_ASM || variant == OPENCNN_KERNEL_AUTO) && !ragged && kw > 1 &&
-      (long long)a.nblocks * (in_c / 8) <= kMaxElems &&
+  const int chunks = (in_c + 7) / 8;
+  if ((variant == OPENCNN_KERNEL_ASM || variant == OPENCNN_KERNEL_AUTO) && kw > 1 &&
+      (long long)a.nblocks * chunks <= kMaxElems &&
       // per-lane store offsets: four filter rows plus one image row and column, in bytes
       ((long long)in_n * in_h * in_w * 4 + (long long)(in_w + 1) * in_n) * 4 <= kMaxElems) {
     int cus_asm = 0;
@@ -275,7 +278,6 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   }
   if (variant == OPENCNN_KERNEL_ASM) REQUIRE(agrid > 0);
   if (agrid > 0) {
-    const int chunks = in_c / 8;
     const AsmKernels* ak = nullptr;
     if (int e = asm_kernels(&ak)) return e;
     AsmKernArgs ka{};
@@ -291,12 +293,14 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
     ka.ngroups = a.ngroups;
     ka.colgroups = a.colgroups;
     ka.colblocks = a.colblocks;
-    ka.Q = in_c / 4;
+    ka.Q = chunks * 2;
     ka.HWN4 = in_n * in_h * in_w * 4;
+    ka.c_real = in_c;
+    ka.k_real = filt_k;
     const long long total = (long long)a.nblocks * chunks;
     ka.units_q = (int32_t)(total / agrid);
     ka.units_rem = (int32_t)(total % agrid);
-    ka.usw_bytes = (int32_t)((long long)in_c * 16 * filt_k * 4);
+    ka.usw_bytes = (int32_t)(padded_c(in_c) * 16 * padded_k(filt_k) * 4);
     ka.grid_per_xcd = agrid % 8 == 0 ? agrid / 8 : 0;  // 0: no XCD-aware block order
     magic_divisor((uint32_t)chunks, &ka.m_chunks, &ka.s_chunks);
     magic_divisor((uint32_t)a.colblocks, &ka.m_colblocks, &ka.s_colblocks);
@@ -305,7 +309,8 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
     size_t ka_size = sizeof(ka);
     void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &ka, HIP_LAUNCH_PARAM_BUFFER_SIZE, &ka_size,
                      HIP_LAUNCH_PARAM_END};
-    return (int)hipModuleLaunchKernel(kw == 4 ? ak->kw4 : ak->kw2, (unsigned)agrid, 1, 1, 256, 1, 1,
+    const hipFunction_t fn = ragged ? (kw == 4 ? ak->kw4_ragged : ak->kw2_ragged) : (kw == 4 ? ak->kw4 : ak->kw2);
+    return (int)hipModuleLaunchKernel(fn, (unsigned)agrid, 1, 1, 256, 1, 1,
                                       (unsigned)lds_bytes, st, nullptr, extra);
   }
   if (kw == 1) {

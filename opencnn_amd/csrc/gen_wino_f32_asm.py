@@ -2,7 +2,7 @@
 """Generator of the hand-scheduled gfx950 assembly of the fused Winograd F(2x2,3x3) kernel.
 
 Emits one kernel per KW (waves of a workgroup that share a column tile): wino_f32_asm_kw2 and
-wino_f32_asm_kw4.  Same mathematics and data layout as wino_f32_stream in
+wino_f32_asm_kw4, each also as a _ragged variant for shapes outside the reference's tiling.  Same mathematics and data layout as wino_f32_stream in
 conv_kernel_f32.hpp (which replaces the reference's Winograd_kernel,
 src/convolutionForward_32x64x8.cu:169-262); what the assembly adds is control over the things
 hipcc does not let the C++ source decide:
@@ -60,14 +60,19 @@ def a(i, n=1):
 
 
 class Kernel:
-    def __init__(self, KW):
+    def __init__(self, KW, ragged=False):
+        """ragged: shapes outside N % 32 == 0, K % 32 == 0, C % 8 == 0.  Groups and chunks are
+        rounded up by the host; lanes whose batch element does not exist read zeros and store
+        nothing (out-of-range offsets), the last channel slab ends with the tensor, filter rows
+        past K fall outside the row's num_records.  The inner loop is the same."""
         self.KW = KW
+        self.ragged = ragged
         self.CW = 4 // KW
         self.SPW = 4 // KW
         self.lines = []
         self.outofline = []  # rarely executed blocks, emitted behind s_endpgm
         self.nlabel = 0
-        self.name = f"wino_f32_asm_kw{KW}"
+        self.name = f"wino_f32_asm_kw{KW}" + ("_ragged" if ragged else "")
         self.alloc()
 
     # ------------------------------------------------------------------ helpers
@@ -92,7 +97,7 @@ class Kernel:
         S.next = 40
         names = ["N", "H", "W", "Chunks", "TilesW", "Ngroups", "Colgroups", "Colblocks", "Q", "HWN4",
                  "UnitsQ", "UnitsRem", "UswBytes", "GridPerXcd", "Mch", "Sch", "Mcb", "Scb", "Mng",
-                 "Sng", "Mtw", "Stw", "Spare0", "Spare1"]
+                 "Sng", "Mtw", "Stw", "Creal", "Kreal"]
         self.S = {n: self.sInt + i for i, n in enumerate(names)}
         self.S.update(X=8, U=10, Y=12, Sync=14)
         for n in ["L", "Kw", "Cw", "Wave", "Begin", "Nunits", "G", "Tp", "Cp", "Tq", "Cq", "Tm", "Cm",
@@ -110,7 +115,7 @@ class Kernel:
         V = Alloc(1, 256)
         self.V = {}
         for n, cnt, al in [("Lane", 1, 1), ("LaneX", 1, 1), ("Lane8", 1, 1), ("Lane8b", 1, 1),
-                           ("Lds", 1, 1), ("LdsWr", 1, 1), ("Zero", 1, 1), ("One", 1, 1), ("Tmp", 4, 1),
+                           ("Lds", 1, 1), ("LdsWr", 1, 1), ("Zero", 1, 1), ("One", 1, 1), ("Oob", 1, 1), ("Tmp", 4, 1),
                            ("Off", 4, 1), ("Eff", 4, 1), ("VOFF", 16, 1),
                            ("U0", 32, 2), ("U1", 32, 2), ("D0", 16, 1), ("D1", 16, 1),
                            ("VA", 16, 2), ("VB", 16, 2), ("T", 16, 2), ("TO", 16, 2), ("MPX", 16, 1)]:
@@ -173,6 +178,8 @@ class Kernel:
         self.e(f"s_add_i32 {t(2)}, {t(2)}, {t(3)}")
         self.e(f"s_lshl_b32 {t(3)}, {self.sr('Dng')}, 7")
         self.e(f"s_add_i32 {t(2)}, {t(2)}, {t(3)}")  # byte offset of element (0,0), may be negative
+        if self.ragged:
+            self.alive_lanes()
         for i in range(4):
             self.e(f"s_add_i32 {t(4)}, {t(0)}, {i}")
             self.e(f"s_cmp_lt_u32 {t(4)}, {self.sr('H')}")  # unsigned: also rejects -1
@@ -185,10 +192,20 @@ class Kernel:
                 self.e(f"s_cmp_lg_u32 {t(4)}, 0")
                 self.e(f"s_cselect_b32 {t(5)}, {t(3)}, 0x{OOB:x}")
                 self.e(f"v_add_u32 {self.vr('VOFF', i * 4 + j)}, {t(5)}, {self.vr('LaneX')}")
+                if self.ragged:
+                    self.e(f"v_cndmask_b32 {self.vr('VOFF', i * 4 + j)}, {self.vr('Oob')}, {self.vr('VOFF', i * 4 + j)}, vcc")
                 if j < 3:
                     self.e(f"s_add_i32 {t(3)}, {t(3)}, {self.sr('ColStep')}")
             if i < 3:
                 self.e(f"s_add_i32 {t(2)}, {t(2)}, {self.sr('RowStep')}")
+
+    def alive_lanes(self):
+        """vcc = lanes whose batch element Dng*32 + lane%32 exists (ragged N)."""
+        t = self.t
+        self.e(f"s_lshl_b32 {t(4)}, {self.sr('Dng')}, 5")
+        self.e(f"v_and_b32 {self.vr('Tmp')}, 31, {self.vr('Lane')}")
+        self.e(f"v_add_u32 {self.vr('Tmp')}, {t(4)}, {self.vr('Tmp')}")
+        self.e(f"v_cmp_gt_u32 vcc, {self.sr('N')}, {self.vr('Tmp')}")
 
     def slab_descriptor(self, j):
         """RsrcX = the two-channel slab of MFMA step Cp*4 + kw*SPW + j."""
@@ -197,9 +214,15 @@ class Kernel:
         self.e(f"s_add_u32 {t(0)}, {t(0)}, {self.sr('KwSpw')}")
         if j:
             self.e(f"s_add_u32 {t(0)}, {t(0)}, {j}")
+        rx = self.S["RsrcX"]
+        if self.ragged:  # channels of this slab that exist: 2, 1 (odd C) or 0 (padding of the last chunk)
+            self.e(f"s_lshl_b32 {t(2)}, {t(0)}, 1")
+            self.e(f"s_sub_i32 {t(2)}, {self.sr('Creal')}, {t(2)}")
+            self.e(f"s_max_i32 {t(2)}, {t(2)}, 0")
+            self.e(f"s_min_i32 {t(2)}, {t(2)}, 2")
+            self.e(f"s_mul_i32 {s(rx + 2)}, {t(2)}, {self.sr('HWN4')}")
         self.e(f"s_mul_hi_u32 {t(1)}, {t(0)}, {self.sr('Slab')}")
         self.e(f"s_mul_i32 {t(0)}, {t(0)}, {self.sr('Slab')}")
-        rx = self.S["RsrcX"]
         self.e(f"s_add_u32 {s(rx)}, {s(self.S['X'])}, {t(0)}")
         self.e(f"s_addc_u32 {s(rx + 1)}, {s(self.S['X'] + 1)}, {t(1)}")
 
@@ -228,10 +251,14 @@ class Kernel:
         self.e(f"s_cmp_lt_u32 {t(1)}, {self.sr('W')}")
         self.e(f"s_cselect_b32 {t(1)}, {self.sr('Dlive')}, 0")  # column 1 stored
         self.e(f"s_and_b32 {t(2)}, {t(0)}, {t(1)}")
+        if self.ragged:
+            self.alive_lanes()
         for q, ok in enumerate([self.sr("Dlive"), t(1), t(0), t(2)]):
             self.e(f"s_cmp_lg_u32 {ok}, 0")
             self.e(f"s_cselect_b32 {t(3)}, 0, 0x{OOB:x}")
             self.e(f"v_or_b32 {self.vr('Eff', q)}, {t(3)}, {self.vr('Off', q)}")
+            if self.ragged:
+                self.e(f"v_cndmask_b32 {self.vr('Eff', q)}, {self.vr('Oob')}, {self.vr('Eff', q)}, vcc")
         # first row of the tile: y + kg*32*HWN4 + ((2ty*W + 2tx)*N + ng*32)*4
         yt = self.S["Yt"]
         self.e(f"s_lshl_b32 {t(0)}, {self.sr('KgM')}, 5")
@@ -402,6 +429,28 @@ class Kernel:
         self.e(f"s_add_u32 {self.sr('Cm')}, {self.sr('Cm')}, 1")
 
     # ------------------------------------------------------------------ epilogue
+    def row_start(self):
+        """RsrcY = first filter row of the tile."""
+        ry = self.S["RsrcY"]
+        self.e(f"s_mov_b32 {s(ry)}, {s(self.S['Yt'])}")
+        self.e(f"s_mov_b32 {s(ry + 1)}, {s(self.S['Yt'] + 1)}")
+        if self.ragged:
+            self.e(f"s_lshl_b32 {self.t(2)}, {self.sr('KgM')}, 5")   # first filter of the wave tile
+            self.e(f"s_lshl_b32 {self.t(3)}, {self.sr('HWN4')}, 2")  # lane offsets below this: hsel = 0
+            self.row_limit(0)
+
+    def row_limit(self, r):
+        """ragged K: num_records of the row descriptor admits the lanes whose filter exists (hsel = 0:
+        filter row, offsets below 4*HWN4; hsel = 1: four rows further, offsets above)."""
+        t = self.t
+        ry = self.S["RsrcY"]
+        self.e(f"s_add_u32 {t(0)}, {t(2)}, {8 * (r >> 2) + (r & 3)}")
+        self.e(f"s_cmp_lt_u32 {t(0)}, {self.sr('Kreal')}")
+        self.e(f"s_cselect_b32 {t(1)}, {t(3)}, 0")
+        self.e(f"s_add_u32 {t(0)}, {t(0)}, 4")
+        self.e(f"s_cmp_lt_u32 {t(0)}, {self.sr('Kreal')}")
+        self.e(f"s_cselect_b32 {s(ry + 2)}, 0x{OOB:x}, {t(1)}")
+
     def row_advance(self, r):
         """RsrcY: filter row 8*(r/4) + r%4 -> the row of r+1 (the 4*hsel part is in the lane offset)."""
         if r == 15:
@@ -411,6 +460,8 @@ class Kernel:
         for _ in range(mult):
             self.e(f"s_add_u32 {s(ry)}, {s(ry)}, {self.sr('HWN4')}")
             self.e(f"s_addc_u32 {s(ry + 1)}, {s(ry + 1)}, 0")
+        if self.ragged:
+            self.row_limit(r + 1)
 
     def epilogue(self, through):
         """Y = A^T M A per accumulator element (order of src/store_and_transform_output_optSTS64.cuh:29-51)
@@ -418,8 +469,7 @@ class Kernel:
         workgroup on another XCD will read)."""
         pol = " sc0 sc1" if through else ""
         ry = self.S["RsrcY"]
-        self.e(f"s_mov_b32 {s(ry)}, {s(self.S['Yt'])}")
-        self.e(f"s_mov_b32 {s(ry + 1)}, {s(self.S['Yt'] + 1)}")
+        self.row_start()
         # the last MFMAs must have written the accumulators before they are read
         self.e("s_nop 15")
         self.e("s_nop 15")
@@ -493,8 +543,7 @@ class Kernel:
         self.e(f"s_branch {poll}")
         self.label(got)
         ry = self.S["RsrcY"]
-        self.e(f"s_mov_b32 {s(ry)}, {s(self.S['Yt'])}")
-        self.e(f"s_mov_b32 {s(ry + 1)}, {s(self.S['Yt'] + 1)}")
+        self.row_start()
         for r in range(16):
             for q in range(4):
                 self.e(f"buffer_load_dword {v(self.MP[r * 4 + q])}, {self.vr('Eff', q)}, {s(ry, 4)}, 0 offen sc0 sc1")
@@ -525,6 +574,7 @@ class Kernel:
         e(f"v_and_b32 {self.vr('Lane')}, 63, {self.vr('Tmp', 1)}")
         e(f"v_mov_b32 {self.vr('Zero')}, 0")
         e(f"v_mov_b32 {self.vr('One')}, 1")
+        e(f"v_mov_b32 {self.vr('Oob')}, 0x{OOB:x}")
         e("s_waitcnt lgkmcnt(0)")
         # only now: a vector instruction that writes an SGPR while scalar loads are still
         # outstanding came back with a corrupted value on this part
@@ -727,7 +777,7 @@ class Kernel:
 
 def main():
     out = ['\t.amdgcn_target "amdgcn-amd-amdhsa--gfx950"', "\t.amdhsa_code_object_version 6"]
-    kernels = [Kernel(2), Kernel(4)]
+    kernels = [Kernel(2), Kernel(4), Kernel(2, ragged=True), Kernel(4, ragged=True)]
     for k in kernels:
         k.emit(out)
     out.append("\t.amdgpu_metadata\n---\namdhsa.kernels:")

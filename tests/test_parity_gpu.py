@@ -357,33 +357,34 @@ def test_shapes_outside_reference_tiling(ocn, oracle, torch_gpu, N, C, H, W, K):
         assert np.array_equal(r.dropin(), y)
 
 
-def test_ragged_shape_on_both_kernel_families(ocn, oracle, torch_gpu):
-    # two filter groups: the LDS kernel by default, the register kernel on request
-    print("ragged variants", flush=True)
-    x, w = make_tensors(ocn, 48, 12, 7, 7, 64, filt="uniform")
+@pytest.mark.parametrize("N,C,H,K", [(48, 12, 7, 64), (100, 20, 13, 100), (33, 8, 30, 128), (7, 5, 6, 40)])
+def test_ragged_shape_on_every_kernel_family(ocn, oracle, torch_gpu, N, C, H, K):
+    # an even number of filter groups: the assembly kernels by default, the HIP LDS and register
+    # kernels on request
+    print(f"ragged variants N={N} C={C} H={H} K={K}", flush=True)
+    x, w = make_tensors(ocn, N, C, H, H, K, filt="uniform")
     r = Runner(ocn, torch_gpu, x, w)
-    y_lds = r.dropin()
     try:
-        ocn.set_kernel_variant(ocn.KERNEL_REGISTER)
-        y_reg = r.dropin()
+        for variant in (ocn.KERNEL_ASM, ocn.KERNEL_HIP, ocn.KERNEL_REGISTER):
+            ocn.set_kernel_variant(variant)
+            check_against_oracle(oracle, r.dropin(), x, w)
     finally:
         ocn.set_kernel_variant(ocn.KERNEL_AUTO)
-    check_against_oracle(oracle, y_lds, x, w)
-    check_against_oracle(oracle, y_reg, x, w)
 
 
 def test_padded_channels_do_not_leak_non_finite_values(ocn, oracle, torch_gpu):
     # C = 5 runs one 8-channel chunk; the three padded channels multiply zeros on BOTH operands,
     # so an infinity in the last real channel must stay confined to the outputs it reaches
     print("ragged inf", flush=True)
-    N, C, H, K = 32, 5, 6, 32
-    x, w = make_tensors(ocn, N, C, H, H, K, filt="uniform")
-    x[C - 1, 2, 2, 3] = np.inf
-    y = Runner(ocn, torch_gpu, x, w).split()
-    bad = ~np.isfinite(y)
-    assert bad[:, :, :, 3].any()
-    bad[:, :, :, 3] = False
-    assert not bad.any()
+    for K in (32, 64):  # register kernel / assembly kernel
+        N, C, H = 32, 5, 6
+        x, w = make_tensors(ocn, N, C, H, H, K, filt="uniform")
+        x[C - 1, 2, 2, 3] = np.inf
+        y = Runner(ocn, torch_gpu, x, w).split()
+        bad = ~np.isfinite(y)
+        assert bad[:, :, :, 3].any()
+        bad[:, :, :, 3] = False
+        assert not bad.any()
 
 
 # ---------------------------------------------------------------- layout shims
