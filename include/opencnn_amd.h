@@ -60,8 +60,9 @@ int opencnn_set_operand_precision(int precision);
 /*
  * Replaces the reference's hidden set-up: the caller-side cudaMemcpyToSymbol uploads of
  * the fragment-address tables (src/openCNN_winograd.cu:319-331).  This library has no
- * such tables; the call checks that the current device is a gfx950 part and returns
- * hipErrorInvalidDevice otherwise.  Calling it is optional.
+ * such tables; the call checks that the current device is a gfx950 part (hipErrorInvalidDevice
+ * otherwise) and loads the embedded code object of the assembly kernels on it, which the first
+ * launch on a device would otherwise do.  Calling it is optional.
  */
 int opencnn_init(void);
 

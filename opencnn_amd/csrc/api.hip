@@ -377,7 +377,10 @@ int opencnn_init(void) {
     t_last_error = "device is not gfx950";
     return (int)hipErrorInvalidDevice;
   }
-  return 0;
+  // load the assembly kernels now rather than inside the first launch (which may sit in a
+  // stream capture or a timed region)
+  const AsmKernels* ak = nullptr;
+  return asm_kernels(&ak);
 }
 
 int opencnn_tiles_dim(int in_w) {
