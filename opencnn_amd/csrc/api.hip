@@ -184,6 +184,147 @@ int launch_transpose(const float* src, float* dst, long long rows, long long col
   return (int)hipGetLastError();
 }
 
+// fp16 / bf16 GEMM operands: 16-channel chunks, LDS kernel only.
+int launch_h16(opencnn::ConvArgs a, int precision, hipStream_t st) {
+  REQUIRE(a.N % 32 == 0);
+  REQUIRE(a.C % 16 == 0);
+  REQUIRE(a.K % 64 == 0);
+  REQUIRE((long long)a.N * a.H * a.W * 4 * 4 <= kMaxElems);  // four-channel window in bytes
+  const int kw = a.K % 128 == 0 ? 4 : 2, cw = 4 / kw;
+  const long long colblocks = (a.colgroups + cw - 1) / cw;
+  const long long nblocks = colblocks * (a.kgroups / kw);
+  REQUIRE(nblocks <= kMaxElems / 8);
+  a.nblocks = (int)nblocks;
+  a.colblocks = (int)colblocks;
+  dim3 grid(((a.nblocks + 7) / 8) * 8), block(256);
+  const size_t lds = (size_t)cw * 3 * 16 * 2 * 4 * 32 * sizeof(unsigned);
+  const bool bf = precision == OPENCNN_BF16;
+  if (kw == 4) {
+    if (bf)
+      opencnn::wino_h16_fused_lds<4, true><<<grid, block, lds, st>>>(a);
+    else
+      opencnn::wino_h16_fused_lds<4, false><<<grid, block, lds, st>>>(a);
+  } else {
+    // 96 KB of LDS: above the 64 KB a kernel gets without asking (gfx950 has 160 KB per CU)
+    const void* fn = bf ? reinterpret_cast<const void*>(&opencnn::wino_h16_fused_lds<2, true>)
+                        : reinterpret_cast<const void*>(&opencnn::wino_h16_fused_lds<2, false>);
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    if (bf)
+      opencnn::wino_h16_fused_lds<2, true><<<grid, block, lds, st>>>(a);
+    else
+      opencnn::wino_h16_fused_lds<2, false><<<grid, block, lds, st>>>(a);
+  }
+  return (int)hipGetLastError();
+}
+
+// Grid of the hand-scheduled kernels for this layer, or 0 when they do not take it.  One
+// persistent launch whose workgroups share the (tile, chunk) units evenly; it needs whole filter
+// blocks (kw > 1) and at least one tile per workgroup (a tile then has at most two contributors).
+int asm_grid(const opencnn::ConvArgs& a, int kw, int* grid) {
+  *grid = 0;
+  const int chunks = (a.C + 7) / 8;
+  if (kw == 1 || (long long)a.nblocks * chunks > kMaxElems) return 0;
+  // per-lane store offsets: four filter rows plus one image row and column, in bytes
+  if (((long long)a.N * a.H * a.W * 4 + (long long)(a.W + 1) * a.N) * 4 > kMaxElems) return 0;
+  int cus = 0;
+  if (int e = compute_units(&cus)) return e;
+  if (a.nblocks < cus)
+    *grid = a.nblocks;  // one tile per workgroup
+  else if (cus % 8 == 0 && cus <= opencnn::kMaxBalancedBlocks &&
+           (a.nblocks % cus == 0 || g_balance.load() != 0))
+    *grid = cus;
+  return 0;
+}
+
+int launch_asm(const opencnn::ConvArgs& a, int kw, int grid, bool ragged, size_t lds_bytes,
+               hipStream_t st) {
+  const AsmKernels* ak = nullptr;
+  if (int e = asm_kernels(&ak)) return e;
+  const int chunks = (a.C + 7) / 8;
+  AsmKernArgs ka{};
+  ka.x = a.x;
+  ka.usw = a.usw;
+  ka.y = a.y;
+  ka.sync = ak->split_sync;
+  ka.N = a.N;
+  ka.H = a.H;
+  ka.W = a.W;
+  ka.chunks = chunks;
+  ka.tiles_w = a.tiles_w;
+  ka.ngroups = a.ngroups;
+  ka.colgroups = a.colgroups;
+  ka.colblocks = a.colblocks;
+  ka.Q = chunks * 2;
+  ka.HWN4 = a.N * a.H * a.W * 4;
+  ka.c_real = a.C;
+  ka.k_real = a.K;
+  const long long total = (long long)a.nblocks * chunks;
+  ka.units_q = (int32_t)(total / grid);
+  ka.units_rem = (int32_t)(total % grid);
+  ka.usw_bytes = (int32_t)(padded_c(a.C) * 16 * padded_k(a.K) * 4);
+  ka.grid_per_xcd = grid % 8 == 0 ? grid / 8 : 0;  // 0: no XCD-aware block order
+  magic_divisor((uint32_t)chunks, &ka.m_chunks, &ka.s_chunks);
+  magic_divisor((uint32_t)a.colblocks, &ka.m_colblocks, &ka.s_colblocks);
+  magic_divisor((uint32_t)a.ngroups, &ka.m_ngroups, &ka.s_ngroups);
+  magic_divisor((uint32_t)a.tiles_w, &ka.m_tiles_w, &ka.s_tiles_w);
+  size_t ka_size = sizeof(ka);
+  void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &ka, HIP_LAUNCH_PARAM_BUFFER_SIZE, &ka_size,
+                   HIP_LAUNCH_PARAM_END};
+  const hipFunction_t fn =
+      ragged ? (kw == 4 ? ak->kw4_ragged : ak->kw2_ragged) : (kw == 4 ? ak->kw4 : ak->kw2);
+  return (int)hipModuleLaunchKernel(fn, (unsigned)grid, 1, 1, 256, 1, 1, (unsigned)lds_bytes, st,
+                                    nullptr, extra);
+}
+
+// The HIP C++ kernels: register variant (kw == 1), LDS variant, and the LDS variant as one
+// continuous pipeline when the balanced split applies.
+int launch_hip(const opencnn::ConvArgs& a, int kw, bool ragged, bool allow_stream, size_t lds_bytes,
+               hipStream_t st) {
+  dim3 grid(((a.nblocks + 7) / 8) * 8), block(256);
+  if (kw == 1) {
+    if (ragged)
+      opencnn::wino_f32_fused<true><<<grid, block, 0, st>>>(a);
+    else
+      opencnn::wino_f32_fused<false><<<grid, block, 0, st>>>(a);
+    return (int)hipGetLastError();
+  }
+  if (ragged) {
+    if (kw == 4)
+      opencnn::wino_f32_fused_lds<4, false, true><<<grid, block, lds_bytes, st>>>(a);
+    else
+      opencnn::wino_f32_fused_lds<2, false, true><<<grid, block, lds_bytes, st>>>(a);
+    return (int)hipGetLastError();
+  }
+  // More tiles than CUs and not a whole number of rounds: one persistent workgroup per CU,
+  // the chunk-units split evenly (every tile then has at most two contributors).
+  int cus = 0;
+  if (int e = compute_units(&cus)) return e;
+  const bool balanced = g_balance.load() != 0 && a.nblocks > cus && a.nblocks % cus != 0 &&
+                        cus % 8 == 0 && cus <= opencnn::kMaxBalancedBlocks &&
+                        (long long)a.nblocks * (a.C / 8) <= kMaxElems;
+  if (balanced) grid = dim3(cus);
+  // The continuous pipeline pays off when a workgroup walks several tiles; for a single tile
+  // per workgroup the plain LDS kernel has less scalar work per load.
+  const bool stream = balanced && allow_stream;
+  if (kw == 4) {
+    if (stream)
+      opencnn::wino_f32_stream<4, true, true><<<grid, block, lds_bytes, st>>>(a);
+    else if (balanced)
+      opencnn::wino_f32_fused_lds<4, true><<<grid, block, lds_bytes, st>>>(a);
+    else
+      opencnn::wino_f32_fused_lds<4, false><<<grid, block, lds_bytes, st>>>(a);
+  } else {
+    if (stream)
+      opencnn::wino_f32_stream<2, true, false><<<grid, block, lds_bytes, st>>>(a);
+    else if (balanced)
+      opencnn::wino_f32_fused_lds<2, true><<<grid, block, lds_bytes, st>>>(a);
+    else
+      opencnn::wino_f32_fused_lds<2, false><<<grid, block, lds_bytes, st>>>(a);
+  }
+  return (int)hipGetLastError();
+}
+
 int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c, int in_h,
                 int in_w, int filt_k, hipStream_t st) {
   REQUIRE(in != nullptr && Ww != nullptr && out != nullptr);
@@ -203,50 +344,16 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   REQUIRE((long long)a.tiles_h * a.tiles_w * a.ngroups <= kMaxElems / 8);
   a.colgroups = a.tiles_h * a.tiles_w * a.ngroups;
   a.kgroups = (filt_k + 31) / 32;
-  const bool ragged = ragged_shape(in_n, in_c, filt_k);
+  a.nblocks = a.colblocks = 0;
   const int precision = g_precision.load();
-  if (precision != OPENCNN_F32) {
-    // fp16 / bf16 GEMM operands: 16-channel chunks, LDS kernel only
-    REQUIRE(in_n % 32 == 0);
-    REQUIRE(in_c % 16 == 0);
-    REQUIRE(filt_k % 64 == 0);
-    REQUIRE((long long)in_n * in_h * in_w * 4 * 4 <= kMaxElems);  // four-channel window in bytes
-    const int hkw = filt_k % 128 == 0 ? 4 : 2, hcw = 4 / hkw;
-    const long long hblocks = (long long)((a.colgroups + hcw - 1) / hcw) * (a.kgroups / hkw);
-    REQUIRE(hblocks <= kMaxElems / 8);
-    a.nblocks = (int)hblocks;
-    a.colblocks = (a.colgroups + hcw - 1) / hcw;
-    dim3 hgrid(((a.nblocks + 7) / 8) * 8), hblock(256);
-    const size_t hlds = (size_t)hcw * 3 * 16 * 2 * 4 * 32 * sizeof(unsigned);
-    const bool bf = precision == OPENCNN_BF16;
-    if (hkw == 4) {
-      if (bf)
-        opencnn::wino_h16_fused_lds<4, true><<<hgrid, hblock, hlds, st>>>(a);
-      else
-        opencnn::wino_h16_fused_lds<4, false><<<hgrid, hblock, hlds, st>>>(a);
-    } else {
-      // 96 KB of LDS: above the 64 KB a kernel gets without asking (gfx950 has 160 KB per CU)
-      const void* fn = bf ? reinterpret_cast<const void*>(&opencnn::wino_h16_fused_lds<2, true>)
-                          : reinterpret_cast<const void*>(&opencnn::wino_h16_fused_lds<2, false>);
-      hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)hlds);
-      if (e != hipSuccess) return (int)e;
-      if (bf)
-        opencnn::wino_h16_fused_lds<2, true><<<hgrid, hblock, hlds, st>>>(a);
-      else
-        opencnn::wino_h16_fused_lds<2, false><<<hgrid, hblock, hlds, st>>>(a);
-    }
-    return (int)hipGetLastError();
-  }
-  // Waves per workgroup that share one column tile (and split its input transform).  A
-  // ragged shape runs the LDS kernel when its (rounded-up) filter groups fill whole workgroups.
-  int kw = 1;
+  if (precision != OPENCNN_F32) return launch_h16(a, precision, st);
+
+  // Waves per workgroup that share one column tile (and split its input transform): as many as
+  // the (rounded-up) filter groups fill whole workgroups of.
+  const bool ragged = ragged_shape(in_n, in_c, filt_k);
   const int variant = g_variant.load();
-  if (variant != OPENCNN_KERNEL_REGISTER) {
-    if (!ragged)
-      kw = filt_k % 128 == 0 ? 4 : (filt_k % 64 == 0 ? 2 : 1);
-    else
-      kw = a.kgroups % 4 == 0 ? 4 : (a.kgroups % 2 == 0 ? 2 : 1);
-  }
+  int kw = 1;
+  if (variant != OPENCNN_KERNEL_REGISTER) kw = a.kgroups % 4 == 0 ? 4 : (a.kgroups % 2 == 0 ? 2 : 1);
   if (variant == OPENCNN_KERNEL_LDS) REQUIRE(kw > 1);
   const int cw = 4 / kw;
   const long long colblocks = (a.colgroups + cw - 1) / cw;
@@ -254,110 +361,15 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   REQUIRE(nblocks <= kMaxElems / 8);
   a.nblocks = (int)nblocks;
   a.colblocks = (int)colblocks;
-  const int per_xcd = (a.nblocks + 7) / 8;
-  dim3 grid(per_xcd * 8), block(256);
   const size_t lds_bytes = (size_t)cw * 2 * 4 * 16 * 64 * sizeof(float);
-  // Hand-scheduled kernels: one persistent launch whose workgroups share the (tile, chunk) units
-  // evenly.  They need whole filter blocks and at least one tile per workgroup (a tile then has
-  // at most two contributors).
-  int agrid = 0;
-  const int chunks = (in_c + 7) / 8;
-  if ((variant == OPENCNN_KERNEL_ASM || variant == OPENCNN_KERNEL_AUTO) && kw > 1 &&
-      (long long)a.nblocks * chunks <= kMaxElems &&
-      // per-lane store offsets: four filter rows plus one image row and column, in bytes
-      ((long long)in_n * in_h * in_w * 4 + (long long)(in_w + 1) * in_n) * 4 <= kMaxElems) {
-    int cus_asm = 0;
-    if (int e = compute_units(&cus_asm)) return e;
-    if (a.nblocks >= cus_asm) {
-      if (cus_asm % 8 == 0 && cus_asm <= opencnn::kMaxBalancedBlocks &&
-          (a.nblocks % cus_asm == 0 || g_balance.load() != 0))
-        agrid = cus_asm;
-    } else {
-      agrid = a.nblocks;  // one tile per workgroup
-    }
+
+  if (variant == OPENCNN_KERNEL_ASM || variant == OPENCNN_KERNEL_AUTO) {
+    int grid = 0;
+    if (int e = asm_grid(a, kw, &grid)) return e;
+    if (grid > 0) return launch_asm(a, kw, grid, ragged, lds_bytes, st);
+    REQUIRE(variant != OPENCNN_KERNEL_ASM);
   }
-  if (variant == OPENCNN_KERNEL_ASM) REQUIRE(agrid > 0);
-  if (agrid > 0) {
-    const AsmKernels* ak = nullptr;
-    if (int e = asm_kernels(&ak)) return e;
-    AsmKernArgs ka{};
-    ka.x = in;
-    ka.usw = Ww;
-    ka.y = out;
-    ka.sync = ak->split_sync;
-    ka.N = in_n;
-    ka.H = in_h;
-    ka.W = in_w;
-    ka.chunks = chunks;
-    ka.tiles_w = a.tiles_w;
-    ka.ngroups = a.ngroups;
-    ka.colgroups = a.colgroups;
-    ka.colblocks = a.colblocks;
-    ka.Q = chunks * 2;
-    ka.HWN4 = in_n * in_h * in_w * 4;
-    ka.c_real = in_c;
-    ka.k_real = filt_k;
-    const long long total = (long long)a.nblocks * chunks;
-    ka.units_q = (int32_t)(total / agrid);
-    ka.units_rem = (int32_t)(total % agrid);
-    ka.usw_bytes = (int32_t)(padded_c(in_c) * 16 * padded_k(filt_k) * 4);
-    ka.grid_per_xcd = agrid % 8 == 0 ? agrid / 8 : 0;  // 0: no XCD-aware block order
-    magic_divisor((uint32_t)chunks, &ka.m_chunks, &ka.s_chunks);
-    magic_divisor((uint32_t)a.colblocks, &ka.m_colblocks, &ka.s_colblocks);
-    magic_divisor((uint32_t)a.ngroups, &ka.m_ngroups, &ka.s_ngroups);
-    magic_divisor((uint32_t)a.tiles_w, &ka.m_tiles_w, &ka.s_tiles_w);
-    size_t ka_size = sizeof(ka);
-    void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &ka, HIP_LAUNCH_PARAM_BUFFER_SIZE, &ka_size,
-                     HIP_LAUNCH_PARAM_END};
-    const hipFunction_t fn = ragged ? (kw == 4 ? ak->kw4_ragged : ak->kw2_ragged) : (kw == 4 ? ak->kw4 : ak->kw2);
-    return (int)hipModuleLaunchKernel(fn, (unsigned)agrid, 1, 1, 256, 1, 1,
-                                      (unsigned)lds_bytes, st, nullptr, extra);
-  }
-  if (kw == 1) {
-    if (ragged)
-      opencnn::wino_f32_fused<true><<<grid, block, 0, st>>>(a);
-    else
-      opencnn::wino_f32_fused<false><<<grid, block, 0, st>>>(a);
-    return (int)hipGetLastError();
-  }
-  // More tiles than CUs and not a whole number of rounds: one persistent workgroup per CU,
-  // the chunk-units split evenly (every tile then has at most two contributors).
-  if (ragged) {
-    if (kw == 4)
-      opencnn::wino_f32_fused_lds<4, false, true><<<grid, block, lds_bytes, st>>>(a);
-    else
-      opencnn::wino_f32_fused_lds<2, false, true><<<grid, block, lds_bytes, st>>>(a);
-    return (int)hipGetLastError();
-  }
-  int cus = 0;
-  if (int e = compute_units(&cus)) return e;
-  const bool balanced = g_balance.load() != 0 && a.nblocks > cus && a.nblocks % cus != 0 &&
-                        cus % 8 == 0 && cus <= opencnn::kMaxBalancedBlocks &&
-                        (long long)a.nblocks * (in_c / 8) <= kMaxElems;
-  if (balanced) grid = dim3(cus);
-  // The continuous pipeline pays off when a workgroup walks several tiles; for a single tile
-  // per workgroup the plain LDS kernel has less scalar work per load.
-  const bool stream = balanced && g_variant.load() != OPENCNN_KERNEL_LDS;
-  if (kw == 4) {
-    if (stream && balanced)
-      opencnn::wino_f32_stream<4, true, true><<<grid, block, lds_bytes, st>>>(a);
-    else if (stream)
-      opencnn::wino_f32_stream<4, false, true><<<grid, block, lds_bytes, st>>>(a);
-    else if (balanced)
-      opencnn::wino_f32_fused_lds<4, true><<<grid, block, lds_bytes, st>>>(a);
-    else
-      opencnn::wino_f32_fused_lds<4, false><<<grid, block, lds_bytes, st>>>(a);
-  } else {
-    if (stream && balanced)
-      opencnn::wino_f32_stream<2, true, false><<<grid, block, lds_bytes, st>>>(a);
-    else if (stream)
-      opencnn::wino_f32_stream<2, false, false><<<grid, block, lds_bytes, st>>>(a);
-    else if (balanced)
-      opencnn::wino_f32_fused_lds<2, true><<<grid, block, lds_bytes, st>>>(a);
-    else
-      opencnn::wino_f32_fused_lds<2, false><<<grid, block, lds_bytes, st>>>(a);
-  }
-  return (int)hipGetLastError();
+  return launch_hip(a, kw, ragged, variant != OPENCNN_KERNEL_LDS, lds_bytes, st);
 }
 
 }  // namespace
