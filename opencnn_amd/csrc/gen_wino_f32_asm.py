@@ -1,11 +1,11 @@
 #!/usr/bin/env python3
 """Generator of the hand-scheduled gfx950 assembly of the fused Winograd F(2x2,3x3) kernel.
 
-Emits one kernel per KW (waves of a workgroup that share a column tile): wino_f32_asm_kw2 and
-wino_f32_asm_kw4, each also as a _ragged variant for shapes outside the reference's tiling.  Same mathematics and data layout as wino_f32_stream in
-conv_kernel_f32.hpp (which replaces the reference's Winograd_kernel,
-src/convolutionForward_32x64x8.cu:169-262); what the assembly adds is control over the things
-hipcc does not let the C++ source decide:
+Emits one kernel per KW (waves of a workgroup that share a column tile), wino_f32_asm_kw2 and
+wino_f32_asm_kw4, each also as a _ragged variant for shapes outside the reference's tiling.
+Same mathematics and data layout as wino_f32_stream in conv_kernel_f32.hpp (which replaces the
+reference's Winograd_kernel, src/convolutionForward_32x64x8.cu:169-262); what the assembly adds
+is control over the things hipcc does not let the C++ source decide:
 
   * all 256 arch VGPRs are assigned by hand (no spills, no copies through accumulator
     registers), so the epilogue and the tile switch cannot disturb the inner loop;
@@ -20,7 +20,28 @@ hipcc does not let the C++ source decide:
     2x2 tile are the images of the Winograd positions (0,0), -(0,3), -(3,0), (3,3)), which
     takes the merge out of the epilogue.
 
-Kernel arguments (one 128-byte block, see KernArgs in api.hip): four pointers (input CHWN,
+Model.  A unit = one 8-channel chunk of one workgroup tile (KW filter groups x 4/KW column
+tiles); unit index = tile * chunks + chunk.  Workgroup L of the persistent grid owns a
+contiguous range of units, at least one tile long, so a tile is shared by at most two
+workgroups: the part that starts inside a tile is its workgroup's FIRST segment (finishes
+early, publishes its partial outputs past the caches and raises a flag), the part that ends
+inside a tile is the other workgroup's LAST segment (merges).  Three cursors walk the range: M
+(the unit being multiplied), Q = M + 1 (filter loads), P = M + 2 (patch loads).
+
+Registers.  a[16p:16p+15] accumulator of Winograd position p (MFMA D layout: register r, lane
+(h, n) = filter row 8*(r/4) + 4h + r%4, batch element n).  U0 / U1: A operands of the two
+filter quads of a chunk, one dwordx2 per position.  D0 (and D1 when a wave owns two steps):
+patches in flight.  VA / VB: B operands of the current / next MFMA step, read from LDS
+V[cw][buf][step][p][lane].  T / TO: transform temporaries.  VOFF: per-lane byte offsets of the
+16 patch elements (out of range = zero padding).  Off / Eff: the four per-lane store offsets
+and their per-tile version (out of range = do not store).
+
+Hazards handled by hand (nothing inserts wait states into assembly): 32 wait states between
+the last MFMA and v_accvgpr_read and between v_accvgpr_write and the next MFMA; s_nop 4
+after v_readfirstlane before the SGPR is used; no vector instruction writes an SGPR while
+scalar loads are outstanding (v_readfirstlane next to s_load returned corrupted values).
+
+Kernel arguments (one 128-byte block, see AsmKernArgs in api.hip): four pointers (input CHWN,
 transformed filter in MFMA order, output KHWN, split-merge flags) and 24 ints.
 
 Usage: gen_wino_f32_asm.py > wino_f32_asm.s
@@ -35,15 +56,16 @@ MERGE_POSITIONS = {0: (0, False), 3: (1, True), 12: (2, True), 15: (3, False)}
 
 
 class Alloc:
+    """Bump allocator of register indices."""
+
     def __init__(self, first, limit):
-        self.next, self.limit, self.names = first, limit, {}
+        self.next, self.limit = first, limit
 
     def get(self, name, n=1, align=1):
         self.next = (self.next + align - 1) // align * align
         base = self.next
         self.next += n
         assert self.next <= self.limit, f"out of registers at {name}"
-        self.names[name] = (base, n)
         return base
 
 
@@ -91,14 +113,13 @@ class Kernel:
 
     # ------------------------------------------------------------------ registers
     def alloc(self):
-        S = Alloc(4, 100)
-        self.sPtr = 8      # s[8:15]: x, usw, y, sync
-        self.sInt = 16     # s[16:39]: the 24 ints
-        S.next = 40
+        # s[0:1] kernel argument pointer, s2 workgroup id, s[8:15] the four pointers,
+        # s[16:39] the 24 ints, s40.. everything else
+        S = Alloc(40, 100)
         names = ["N", "H", "W", "Chunks", "TilesW", "Ngroups", "Colgroups", "Colblocks", "Q", "HWN4",
                  "UnitsQ", "UnitsRem", "UswBytes", "GridPerXcd", "Mch", "Sch", "Mcb", "Scb", "Mng",
                  "Sng", "Mtw", "Stw", "Creal", "Kreal"]
-        self.S = {n: self.sInt + i for i, n in enumerate(names)}
+        self.S = {n: 16 + i for i, n in enumerate(names)}
         self.S.update(X=8, U=10, Y=12, Sync=14)
         for n in ["L", "Kw", "Cw", "Wave", "Begin", "Nunits", "G", "Tp", "Cp", "Tq", "Cq", "Tm", "Cm",
                   "SegEnd", "Kind", "KgM", "KgQ", "ColStep", "RowStep", "Slab", "UoffM", "UoffQ",
@@ -115,7 +136,8 @@ class Kernel:
         V = Alloc(1, 256)
         self.V = {}
         for n, cnt, al in [("Lane", 1, 1), ("LaneX", 1, 1), ("Lane8", 1, 1), ("Lane8b", 1, 1),
-                           ("Lds", 1, 1), ("LdsWr", 1, 1), ("Zero", 1, 1), ("One", 1, 1), ("Oob", 1, 1), ("Tmp", 4, 1),
+                           ("Lds", 1, 1), ("LdsWr", 1, 1), ("Zero", 1, 1), ("One", 1, 1), ("Oob", 1, 1),
+                           ("Tmp", 4, 1),
                            ("Off", 4, 1), ("Eff", 4, 1), ("VOFF", 16, 1),
                            ("U0", 32, 2), ("U1", 32, 2), ("D0", 16, 1), ("D1", 16, 1),
                            ("VA", 16, 2), ("VB", 16, 2), ("T", 16, 2), ("TO", 16, 2), ("MPX", 16, 1)]:
