@@ -452,6 +452,8 @@ REL_L2_QUANTISED_RESTATEMENT = 2e-5
     (32, 16, 7, 64, (-1.0, 1.0)),      # odd size, two waves per column tile
     (64, 48, 9, 128, (0.0, 1.0)),      # odd number of 16-channel chunks
     (32, 32, 4, 192, (-1.0, 1.0)),
+    (64, 32, 40, 128, (-1.0, 1.0)),    # 800 workgroup tiles of two chunks: tiles cut between workgroups
+    (32, 48, 45, 64, (-1.0, 1.0)),     # the same with a missing column tile and three chunks
 ])
 def test_reduced_precision_operands(ocn, oracle, torch_gpu, prec, N, C, H, K, xr):
     print(f"reduced {prec} N={N} C={C} H={H} K={K}", flush=True)
