@@ -501,5 +501,48 @@ def test_non_default_stream(ocn, oracle, torch_gpu):
     check_against_oracle(oracle, y, x, w)
 
 
+@pytest.mark.parametrize("N,C,H,K", [(32, 8, 8, 64), (64, 16, 40, 128)])
+def test_call_replays_from_a_captured_graph(ocn, oracle, torch_gpu, N, C, H, K):
+    # The drop-in call only launches kernels (no allocation, no memset, its device state resets
+    # itself), so it can be captured; the second shape has tiles cut between workgroups.  Replays
+    # with new inputs, eager launches and synchronisations in between, each checked.
+    print(f"graph N={N} C={C} H={H} K={K}", flush=True)
+    torch = torch_gpu
+    ocn.init()  # loads the assembly kernels' code object outside the capture
+    x, w = make_tensors(ocn, N, C, H, H, K)
+    r = Runner(ocn, torch, x, w)
+    td = ocn.tiles_dim(H)
+
+    def launch():
+        ocn.convolutionForward(r.xd, H, H, r.wd, H, H, N, K, r.yd, r.ws, r.n_out, td, N, 4, td * 4,
+                               C, K, C, 3, 3, 4, 2)
+
+    s = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    try:
+        ocn.set_stream(s)
+        with torch.cuda.stream(s):
+            launch()
+            s.synchronize()
+            with torch.cuda.graph(g, stream=s):
+                launch()
+        for rep in range(3):
+            x2, w2 = ocn.synth_input(N, C, H, H, seed=100 + rep), ocn.synth_filter(K, C, seed=200 + rep)
+            r.xd.copy_(torch.from_numpy(x2).to(r.xd.device))
+            r.wd.copy_(torch.from_numpy(w2).to(r.wd.device))
+            r.raw.fill_(float("nan"))
+            torch.cuda.synchronize()
+            g.replay()
+            y_graph = r.result()
+            with torch.cuda.stream(s):
+                launch()
+            y_eager = r.result()
+            assert np.array_equal(y_graph, y_eager)
+            check_against_oracle(oracle, y_graph, x2, w2)
+    finally:
+        ocn.set_stream(None)
+
+
 def test_init_accepts_this_device(ocn, torch_gpu):
     ocn.init()
