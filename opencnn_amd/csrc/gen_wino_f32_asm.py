@@ -331,27 +331,63 @@ class Kernel:
         o = lambda i: self.vr("TO", i)
         self.e(f"ds_write2st64_b32 {self.vr('LdsWr')}, {o(p)}, {o(p + 1)} offset0:{j * 16 + p} offset1:{j * 16 + p + 1}")
 
-    def mfma_step(self, step, first, vmem, scalar_work=None, write_step=None):
-        """16 MFMAs of one step; behind MFMA p: vmem(p) (one global load or nothing) and, for
-        p < 8, the LDS read of two B operands of the next step.  scalar_work() is emitted behind
-        the first MFMA: scalar instructions issue while the matrix pipe is busy.  write_step: the
-        transformed patch waiting in TO goes to LDS as owned step `write_step`, two values
-        behind each of the first eight MFMAs."""
+    def mfma_slot(self, step, first, p, vmem, write_step):
+        """MFMA p of a step and what rides behind it: vmem(p) (global loads or nothing), for
+        p < 8 the LDS read of two B operands of the next step and, with write_step, the LDS write
+        of two transformed values waiting in TO (owned step `write_step`)."""
         usrc = "U0" if step < 2 else "U1"
         vsrc = "VA" if step % 2 == 0 else "VB"
         vnext = "VB" if step % 2 == 0 else "VA"
+        fresh = first and step == 0 and not (first == "merge" and p in MERGE_POSITIONS)
+        c = "0" if fresh else a(16 * p, 16)
+        self.e(f"v_mfma_f32_32x32x2_f32 {a(16 * p, 16)}, {self.vr(usrc, 2 * p + (step & 1))}, {self.vr(vsrc, p)}, {c}")
+        if vmem:
+            vmem(p)
+        if step < 3 and p < 8:
+            self.read_v(vnext, step + 1, 2 * p)
+        if write_step is not None and p < 8:
+            self.write_v(write_step, 2 * p)
+
+    def mfma_step(self, step, first, vmem, write_step=None):
+        """The 16 MFMAs of one step."""
         for p in range(16):
-            fresh = first and step == 0 and not (first == "merge" and p in MERGE_POSITIONS)
-            c = "0" if fresh else a(16 * p, 16)
-            self.e(f"v_mfma_f32_32x32x2_f32 {a(16 * p, 16)}, {self.vr(usrc, 2 * p + (step & 1))}, {self.vr(vsrc, p)}, {c}")
-            if vmem:
-                vmem(p)
-            if step < 3 and p < 8:
-                self.read_v(vnext, step + 1, 2 * p)
-            if write_step is not None and p < 8:
-                self.write_v(write_step, 2 * p)
-            if p == 0 and scalar_work:
-                scalar_work()
+            self.mfma_slot(step, first, p, vmem, write_step)
+
+    def mfma_step_with_cursors(self, first, vmem, write_step):
+        """Step 0, during which the cursors P and Q advance: scalar instructions issue while the
+        matrix pipe is busy, in front of the chunk it would wait for them.  The common case (P
+        stays in its tile) is a handful of instructions behind the first MFMA, without a taken
+        branch.  The tile switch of P (three divisions, 16 patch offsets: some 150 instructions)
+        is a second copy of the rest of the step, out of line behind the kernel's end, with the
+        switch spread over the gaps between its MFMAs."""
+        t = self.t
+        rare, done = self.newlabel("p_switch"), self.newlabel("step0_done")
+        self.mfma_slot(0, first, 0, vmem, write_step)
+        self.e(f"s_add_u32 {t(0)}, {self.sr('G')}, 2")
+        self.e(f"s_cmp_lt_u32 {t(0)}, {self.sr('Nunits')}")
+        self.e(f"s_addc_u32 {self.sr('Cp')}, {self.sr('Cp')}, 0")  # P -> unit G+2 when there is one
+        self.e(f"s_cmp_eq_u32 {self.sr('Cp')}, {self.sr('Chunks')}")
+        self.e(f"s_cbranch_scc1 {rare}")
+        self.advance_q()
+        for p in range(1, 16):
+            self.mfma_slot(0, first, p, vmem, write_step)
+        self.label(done)
+        # the rare path
+        main, self.lines = self.lines, []
+        self.e(f"s_mov_b32 {self.sr('Cp')}, 0")
+        self.e(f"s_add_u32 {self.sr('Tp')}, {self.sr('Tp')}, 1")
+        self.decode(self.sr("Tp"))
+        self.patch_offsets()
+        switch, self.lines = self.lines, []
+        self.label(rare)
+        self.advance_q()  # first: it shares the scalar temporaries with the switch
+        per_gap = -(-len(switch) // 15)
+        for p in range(1, 16):
+            self.lines.extend(switch[(p - 1) * per_gap:p * per_gap])
+            self.mfma_slot(0, first, p, vmem, write_step)
+        self.e(f"s_branch {done}")
+        self.outofline.extend(self.lines)
+        self.lines = main
 
     def end_of_chunk(self):
         """All LDS traffic of this wave done, workgroup barrier, swap the buffers, fetch the first
@@ -423,12 +459,7 @@ class Kernel:
         self.u_offset(self.sr("UoffM"), self.sr("KgM"), self.sr("Cm"), True)
         wait(16 if two else 0)  # U0 of this unit has landed
         self.e("s_waitcnt lgkmcnt(0)")  # first B operands
-        # The cursors move behind the first MFMA (the patch loads of step 1 and the filter loads
-        # of step 2 are their first users); in front of the chunk the matrix pipe would wait.
-        def cursors():
-            self.advance_p()
-            self.advance_q()
-        self.mfma_step(0, first, lambda p: self.load_u("U1", p, self.sr("UoffM")), cursors, write_step=0)
+        self.mfma_step_with_cursors(first, lambda p: self.load_u("U1", p, self.sr("UoffM")), write_step=0)
         # step 1
         self.slab_descriptor(0)
         self.e("s_waitcnt lgkmcnt(0)")

@@ -43,10 +43,12 @@ def test_kernel_text_invariants(gen, kw):
     text = "\n".join(k.lines)
     # one workgroup barrier per chunk variant + the prologue; three chunk variants
     assert text.count("s_barrier") == 4
-    # 64 MFMAs per chunk variant
-    assert len(re.findall(r"v_mfma_f32_32x32x2_f32", text)) == 3 * 64
-    # first step of a tile: 16 MFMAs from the constant 0; a merging segment keeps four accumulators
-    assert len(re.findall(r"v_mfma_f32_32x32x2_f32 [^\n]*, 0$", text, re.M)) == 16 + 12
+    # 64 MFMAs per chunk variant, plus the second copy of step 0 (MFMAs 1..15) that carries the
+    # tile switch of the patch cursor
+    assert len(re.findall(r"v_mfma_f32_32x32x2_f32", text)) == 3 * (64 + 15)
+    # first step of a tile: 16 MFMAs from the constant 0 (15 in the second copy); a merging segment
+    # keeps four accumulators (three of them among MFMAs 1..15)
+    assert len(re.findall(r"v_mfma_f32_32x32x2_f32 [^\n]*, 0$", text, re.M)) == (16 + 15) + (12 + 12)
     # the counted waits rely on exactly 64 stores per epilogue (two epilogues: plain, publishing)
     assert len(re.findall(r"buffer_store_dword", text)) == 2 * 64
     assert len(re.findall(r"buffer_store_dword [^\n]* sc0 sc1", text)) == 64
