@@ -501,6 +501,54 @@ def test_non_default_stream(ocn, oracle, torch_gpu):
     check_against_oracle(oracle, y, x, w)
 
 
+def test_random_shapes_on_every_kernel_family(ocn, oracle, torch_gpu):
+    # seeded sweep over batch sizes, channel and filter counts inside and outside the reference's
+    # tiling, square and rectangular images, default / HIP-only kernels, balanced split on / off:
+    # every output element written exactly inside the tensor, two calls bit-identical, rel-L2
+    # against the fp64 direct convolution
+    import random
+
+    torch = torch_gpu
+    rng = random.Random(20241)
+    guard = 4096
+    for case in range(48):
+        N = rng.choice([1, 5, 16, 31, 32, 33, 48, 64, 96, 100, 128])
+        C = rng.choice([1, 3, 7, 8, 9, 16, 20, 24, 40, 64, 72])
+        H = rng.randint(1, 48)
+        W = rng.choice([H, H, rng.randint(1, 48)])
+        K = rng.choice([8, 32, 40, 64, 64, 96, 100, 128, 128, 192, 250, 256])
+        if N * C * H * W * K * 18 > 8e9:
+            continue
+        variant = rng.choice([ocn.KERNEL_AUTO, ocn.KERNEL_AUTO, ocn.KERNEL_HIP])
+        balanced = rng.random() < 0.8
+        print(f"random case {case}: N={N} C={C} H={H} W={W} K={K} variant={variant} balanced={balanced}", flush=True)
+        x = ocn.synth_input(N, C, H, W, seed=case + 1)
+        w = ocn.synth_filter(K, C, seed=case + 1000, dist=ocn.DIST_UNIFORM, p0=-1.0, p1=1.0)
+        xd, wd = torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda()
+        raw = torch.full((K * H * W * N + 2 * guard,), float("nan"), device="cuda")
+        y = raw[guard:guard + K * H * W * N]
+        ws = torch.full((ocn.workspace_bytes(C, K) // 4,), float("nan"), device="cuda")
+        runs = []
+        try:
+            ocn.set_kernel_variant(variant)
+            ocn.set_balanced_split(balanced)
+            ocn.filter_transform(wd, ws, K, C, ocn.FILTER_CRSK, ocn.WW_MFMA)
+            for _ in range(2):
+                raw.fill_(float("nan"))
+                ocn.conv_forward_pretransformed(xd, ws, y, N, C, H, W, K)
+                torch.cuda.synchronize()
+                runs.append(raw.cpu().numpy().copy())
+        finally:
+            ocn.set_kernel_variant(ocn.KERNEL_AUTO)
+            ocn.set_balanced_split(True)
+        assert np.isnan(runs[0][:guard]).all() and np.isnan(runs[0][-guard:]).all(), "wrote outside the output"
+        got = runs[0][guard:-guard]
+        assert not np.isnan(got).any(), "an output element was never written"
+        assert np.array_equal(got, runs[1][guard:-guard])
+        rel64, _, _ = oracle.compare(got.reshape(K, H, W, N), oracle.direct_conv_f64(x, w))
+        assert rel64 <= 1e-5, f"rel-L2 vs fp64 direct {rel64:.3e}"
+
+
 @pytest.mark.parametrize("N,C,H,K", [(32, 8, 8, 64), (64, 16, 40, 128)])
 def test_call_replays_from_a_captured_graph(ocn, oracle, torch_gpu, N, C, H, K):
     # The drop-in call only launches kernels (no allocation, no memset, its device state resets
