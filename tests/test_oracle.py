@@ -1,6 +1,7 @@
 """Pins the CPU oracle against what the mathematics fixes (the reference ships no tests,
 fixtures or golden vectors for this path): closed forms in fp64, textbook matrices,
 brute force on tiny inputs, exact-integer cases where every summation order agrees."""
+import os
 import numpy as np
 import pytest
 
@@ -179,3 +180,20 @@ def test_quantised_restatement_vs_direct(oracle, quant, bound):
     w = rng.normal(0, np.sqrt(2.0 / (9 * C)), (C, 3, 3, K)).astype(np.float32)
     rel, _, _ = oracle.compare(oracle.winograd_f32(x, w, quant), oracle.direct_conv_f64(x, w))
     assert 1e-6 < rel <= bound  # quantisation visible, inside the stated bound
+
+
+# ---------------------------------------------------------------- committed known-answer vectors
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+GOLDEN_CASES = sorted(f[:-4] for f in os.listdir(GOLDEN) if f.endswith(".npz"))
+
+
+@pytest.mark.parametrize("name", GOLDEN_CASES)
+def test_oracle_reproduces_known_answer_vectors(oracle, name):
+    # tests/golden/*.npz: integer tensors and their exact int64 convolution (numpy only,
+    # tests/golden/make_vectors.py); both oracle paths must hit them bit for bit
+    v = np.load(os.path.join(GOLDEN, name + ".npz"))
+    x, w, y = v["x"].astype(np.float32), v["w"].astype(np.float32), v["y"]
+    assert np.array_equal(oracle.direct_conv_f64(x, w), y.astype(np.float64))
+    if x.shape[1] == x.shape[2]:  # the restatement follows the reference: square images only
+        assert np.array_equal(oracle.winograd_f32(x, w), y.astype(np.float32))

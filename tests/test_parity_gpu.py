@@ -4,6 +4,8 @@ Tolerances (fp32 path): relative L2 <= 1e-5 and max-abs <= 1e-4 * max|y| against
 reference-order fp32 Winograd restatement; relative L2 <= 1e-3 against the fp64 direct
 convolution.  Filter transform and exact-integer cases: bit-exact.
 """
+import os
+
 import numpy as np
 import pytest
 
@@ -172,6 +174,27 @@ def test_integer_tensors_bit_exact(ocn, oracle, torch_gpu):
     y = Runner(ocn, torch_gpu, x, w).dropin()
     assert np.array_equal(y.astype(np.float64), oracle.direct_conv_f64(x, w))
     assert np.array_equal(y, oracle.winograd_f32(x, w))
+
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+GOLDEN_CASES = sorted(f[:-4] for f in os.listdir(GOLDEN) if f.endswith(".npz"))
+
+
+@pytest.mark.parametrize("family", ["auto", "hip", "register"])
+@pytest.mark.parametrize("name", GOLDEN_CASES)
+def test_known_answer_vectors_bit_exact(ocn, torch_gpu, name, family):
+    # committed integer tensors with their exact convolution (tests/golden/make_vectors.py, numpy
+    # only): every kernel family must reproduce them bit for bit, whatever its summation order
+    print(f"golden {name} {family}", flush=True)
+    v = np.load(os.path.join(GOLDEN, name + ".npz"))
+    x, w, want = v["x"].astype(np.float32), v["w"].astype(np.float32), v["y"].astype(np.float32)
+    r = Runner(ocn, torch_gpu, x, w)
+    try:
+        ocn.set_kernel_variant({"auto": ocn.KERNEL_AUTO, "hip": ocn.KERNEL_HIP, "register": ocn.KERNEL_REGISTER}[family])
+        y = r.split()
+    finally:
+        ocn.set_kernel_variant(ocn.KERNEL_AUTO)
+    assert np.array_equal(y, want)
 
 
 def test_impulse_reproduces_filter_taps(ocn, torch_gpu):
