@@ -106,6 +106,46 @@ def miopen_column(torch, lay, warmup=10, iters=50):
     return ev[0].elapsed_time(ev[1]) / iters
 
 
+def timeline_summary(ocn, torch, lay, launches=20):
+    """Where a launch of the assembly kernels spends its time: per-workgroup stamps (kernel start,
+    end of the prologue, before / after every output transform) of the last of `launches`
+    back-to-back launches with pre-transformed filters, summarised in microseconds."""
+    import numpy as np
+
+    o = lay
+    ocn.filter_transform(o.w, o.ws, o.K, o.C, ocn.FILTER_CRSK, ocn.WW_MFMA)
+    buf = torch.zeros(1024 * 64, dtype=torch.int64, device=o.x.device)
+    try:
+        ocn.set_timeline_buffer(buf)
+        for _ in range(launches):
+            ocn.conv_forward_pretransformed(o.x, o.ws, o.y, o.N, o.C, o.H, o.H, o.K)
+        torch.cuda.synchronize()
+    finally:
+        ocn.set_timeline_buffer(None)
+    nwg = int((buf.cpu().numpy().reshape(-1, 64)[:, 0] > 0).sum())
+    if nwg == 0:
+        return {"workload": o.name, "recorded_workgroups": 0}
+    t = [np.array(v) for v in ocn.read_timeline(buf, nwg)]
+    ends = np.array([v[-1] for v in t])
+    segs, epis = [], []
+    for v in t:
+        d = np.diff(v)          # prologue, then (segment, output transform) pairs
+        segs += d[1::2].tolist()
+        epis += d[2::2].tolist()
+    segs, epis = np.array(segs), np.array(epis)
+    chunks = o.C // 8
+    return {
+        "workload": o.name, "recorded_workgroups": nwg,
+        "kernel_span_us": float(ends.max()),
+        "workgroup_end_us": {"min": float(ends.min()), "mean": float(ends.mean()), "max": float(ends.max())},
+        "prologue_us_mean": float(np.mean([v[1] - v[0] for v in t])),
+        "whole_tile_us_median": float(np.median(segs[segs > 0.75 * segs.max()])),
+        "chunks_per_tile": chunks,
+        "output_transform_us_median": float(np.median(epis)),
+        "segments_per_workgroup_mean": float(np.mean([(len(v) - 2) // 2 for v in t])),
+    }
+
+
 def cpu_baseline(layer):
     """The oracle's fp64 direct convolution on the host cores, one warm + one timed pass."""
     from oracle import oracle
@@ -137,6 +177,9 @@ def main():
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(FP32_LAYERS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-layers", action="store_true", help="skip the per-layer table")
+    ap.add_argument("--timeline", action="store_true",
+                    help="add the assembly kernels' per-workgroup timeline of the workload (and of every "
+                         "fp32 layer of the table) to the output")
     ap.add_argument("--miopen", action="store_true",
                     help="add an informational MIOpen (torch conv2d, fp32) column to the per-layer table")
     args = ap.parse_args()
@@ -214,6 +257,9 @@ def main():
         if not rel <= 1e-3:
             sys.exit(f"bench.py: GPU result differs from the fp64 direct convolution (rel-L2 {rel})")
 
+    if args.timeline:
+        out["timeline"] = [timeline_summary(ocn, torch, layer)]
+
     if not args.no_layers:
         rows = []
         for name in LAYERS:
@@ -240,6 +286,8 @@ def main():
                     "mfma_frac_of_peak": m / (mn * 1e-3) / 1e12 / peak,
                     "hbm_gbs_at_min_bytes": b / (tot * 1e-3) / 1e9,
                 })
+            if args.timeline and name != layer.name and not name.startswith("reduced"):
+                out["timeline"].append(timeline_summary(ocn, torch, lay))
             del lay
         out["layers"] = rows
 

@@ -198,6 +198,16 @@ int opencnn_time_forward(const float *in, const float *w, float *out, float *Ww,
                          int iters, float *ms_total, float *ms_main, float *ms_fx);
 
 /*
+ * Bench support without a counterpart in the reference: a timeline of the assembly kernels.
+ * While a buffer is set, the first wave of workgroup L of every later launch of those kernels
+ * writes into device_buffer[L*64 ...]: [0] the number of stamps, [2], [3], ... the GPU's
+ * 100 MHz realtime counter at kernel start, after the prologue, and before and after every output
+ * transform (at most 62 stamps).  `bytes` is the size of the buffer; launches with more
+ * workgroups than it holds records for do not record.  NULL / 0 turns it off (the default).
+ */
+int opencnn_set_timeline_buffer(long long *device_buffer, size_t bytes);
+
+/*
  * Layout shims on the selected stream, device to device, src != dst: the reference's data_cpy
  * kernel (src/openCNN_winograd.cu:147-153) as used at :230 (NCHW input -> CHWN) and :235 (KCRS
  * filters -> CRSK), plus the way back for the result (KHWN -> NKHW, i.e. NCHW with K channels),

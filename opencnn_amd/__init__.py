@@ -19,6 +19,8 @@ from .binding import (  # noqa: F401
     set_stream,
     set_kernel_variant,
     set_balanced_split,
+    set_timeline_buffer,
+    read_timeline,
     nchw_to_chwn,
     khwn_to_nkhw,
     kcrs_to_crsk,

@@ -45,6 +45,7 @@ EXPORTED_SYMBOLS = {
     "opencnn_set_stream": (_c_int, [_c_void_p]),
     "opencnn_set_kernel_variant": (_c_int, [_c_int]),
     "opencnn_set_balanced_split": (_c_int, [_c_int]),
+    "opencnn_set_timeline_buffer": (_c_int, [_c_void_p, ctypes.c_size_t]),
     "opencnn_set_operand_precision": (_c_int, [_c_int]),
     "opencnn_filter_transform": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int]),
     "opencnn_conv_forward_pretransformed": (
@@ -174,6 +175,27 @@ def set_balanced_split(enable: bool) -> None:
     """Persistent, evenly split launch of the LDS kernel for tile counts that do not fill
     whole rounds of CUs (default on)."""
     _check("opencnn_set_balanced_split", lib().opencnn_set_balanced_split(1 if enable else 0))
+
+
+def set_timeline_buffer(buf) -> None:
+    """Record the assembly kernels' timeline into `buf` (a CUDA int64 tensor with 64 entries per
+    workgroup), or stop recording with None."""
+    if buf is None:
+        _check("opencnn_set_timeline_buffer", lib().opencnn_set_timeline_buffer(None, 0))
+        return
+    if not (buf.is_cuda and buf.is_contiguous() and buf.element_size() == 8):
+        raise ValueError("timeline buffer must be a contiguous CUDA int64 tensor")
+    _check("opencnn_set_timeline_buffer",
+           lib().opencnn_set_timeline_buffer(buf.data_ptr(), buf.numel() * 8))
+
+
+def read_timeline(buf, n_workgroups: int):
+    """Host copy of a recorded timeline: list (one entry per workgroup) of microsecond offsets from
+    the earliest stamp of the launch."""
+    d = buf.cpu().numpy().reshape(-1, 64)[:n_workgroups]
+    counts = d[:, 0].astype(int)
+    t0 = min(int(d[b, 2]) for b in range(n_workgroups) if counts[b] > 0)
+    return [((d[b, 2:2 + counts[b]] - t0) / 100.0).tolist() for b in range(n_workgroups)]
 
 
 def set_operand_precision(precision: int) -> None:

@@ -22,6 +22,8 @@ std::atomic<hipStream_t> g_stream{nullptr};
 std::atomic<int> g_variant{OPENCNN_KERNEL_AUTO};
 std::atomic<int> g_balance{1};
 std::atomic<int> g_precision{OPENCNN_F32};
+std::atomic<long long*> g_timeline{nullptr};
+std::atomic<size_t> g_timeline_bytes{0};
 
 // Compute units of the current device (cached per device index).
 int compute_units(int* out) {
@@ -75,7 +77,7 @@ int asm_kernels(const AsmKernels** out) {
   return 0;
 }
 
-// Argument block of the assembly kernels (128 bytes, the layout gen_wino_f32_asm.py loads).
+// Argument block of the assembly kernels (136 bytes, the layout gen_wino_f32_asm.py loads).
 struct AsmKernArgs {
   const float* x;
   const float* usw;
@@ -85,8 +87,9 @@ struct AsmKernArgs {
   int32_t Q, HWN4, units_q, units_rem, usw_bytes, grid_per_xcd;
   uint32_t m_chunks, s_chunks, m_colblocks, s_colblocks, m_ngroups, s_ngroups, m_tiles_w, s_tiles_w;
   int32_t c_real, k_real;  // read by the _ragged kernels only
+  long long* timeline;     // 64 entries per workgroup, or null
 };
-static_assert(sizeof(AsmKernArgs) == 128, "kernel argument block");
+static_assert(sizeof(AsmKernArgs) == 136, "kernel argument block");
 
 // x / d == (x * m) >> s for 0 <= x < 2^31 (round-up method, 31-bit dividends).
 void magic_divisor(uint32_t d, uint32_t* m, uint32_t* s) {
@@ -264,6 +267,7 @@ int launch_asm(const opencnn::ConvArgs& a, int kw, int grid, bool ragged, size_t
   ka.units_rem = (int32_t)(total % grid);
   ka.usw_bytes = (int32_t)(padded_c(a.C) * 16 * padded_k(a.K) * 4);
   ka.grid_per_xcd = grid % 8 == 0 ? grid / 8 : 0;  // 0: no XCD-aware block order
+  ka.timeline = (size_t)grid * 64 * sizeof(long long) <= g_timeline_bytes.load() ? g_timeline.load() : nullptr;
   magic_divisor((uint32_t)chunks, &ka.m_chunks, &ka.s_chunks);
   magic_divisor((uint32_t)a.colblocks, &ka.m_colblocks, &ka.s_colblocks);
   magic_divisor((uint32_t)a.ngroups, &ka.m_ngroups, &ka.s_ngroups);
@@ -435,6 +439,14 @@ int opencnn_kcrs_to_crsk(const float* src, float* dst, int k, int c) {
 int opencnn_set_operand_precision(int precision) {
   REQUIRE(precision == OPENCNN_F32 || precision == OPENCNN_F16 || precision == OPENCNN_BF16);
   g_precision.store(precision);
+  return 0;
+}
+
+int opencnn_set_timeline_buffer(long long* device_buffer, size_t bytes) {
+  REQUIRE((device_buffer == nullptr) == (bytes == 0));
+  g_timeline_bytes.store(0);
+  g_timeline.store(device_buffer);
+  g_timeline_bytes.store(bytes);
   return 0;
 }
 

@@ -41,8 +41,11 @@ the last MFMA and v_accvgpr_read and between v_accvgpr_write and the next MFMA; 
 after v_readfirstlane before the SGPR is used; no vector instruction writes an SGPR while
 scalar loads are outstanding (v_readfirstlane next to s_load returned corrupted values).
 
-Kernel arguments (one 128-byte block, see AsmKernArgs in api.hip): four pointers (input CHWN,
-transformed filter in MFMA order, output KHWN, split-merge flags) and 24 ints.
+Kernel arguments (one 136-byte block, see AsmKernArgs in api.hip): four pointers (input CHWN,
+transformed filter in MFMA order, output KHWN, split-merge flags), 24 ints and the timeline
+buffer (or null): 64 int64 per workgroup, [0] = number of stamps, [2..] = the 100 MHz realtime
+counter at kernel start, after the prologue and before / after every output transform, taken
+by the workgroup's first wave.
 
 Usage: gen_wino_f32_asm.py > wino_f32_asm.s
 """
@@ -114,11 +117,11 @@ class Kernel:
     # ------------------------------------------------------------------ registers
     def alloc(self):
         # s[0:1] kernel argument pointer, s2 workgroup id, s[8:15] the four pointers,
-        # s[16:39] the 24 ints, s40.. everything else
-        S = Alloc(40, 100)
+        # s[16:39] the 24 ints, s[40:41] the timeline pointer, s42.. everything else
+        S = Alloc(42, 102)
         names = ["N", "H", "W", "Chunks", "TilesW", "Ngroups", "Colgroups", "Colblocks", "Q", "HWN4",
                  "UnitsQ", "UnitsRem", "UswBytes", "GridPerXcd", "Mch", "Sch", "Mcb", "Scb", "Mng",
-                 "Sng", "Mtw", "Stw", "Creal", "Kreal"]
+                 "Sng", "Mtw", "Stw", "Creal", "Kreal", "Timeline", "TimelineHi"]
         self.S = {n: 16 + i for i, n in enumerate(names)}
         self.S.update(X=8, U=10, Y=12, Sync=14)
         for n in ["L", "Kw", "Cw", "Wave", "Begin", "Nunits", "G", "Tp", "Cp", "Tq", "Cq", "Tm", "Cm",
@@ -614,6 +617,37 @@ class Kernel:
         self.e("s_nop 15")
         self.e("s_nop 15")
 
+    def stamp(self):
+        """Timeline: the workgroup's first wave appends the realtime counter to its 64-entry record
+        (when a buffer was given and the record has room).  The stamp count lives in the register
+        that held Begin during set-up."""
+        t = self.t
+        skip = self.newlabel("no_stamp")
+        tl = self.S["Timeline"]
+        self.e(f"s_cmp_eq_u64 {s(tl, 2)}, 0")
+        self.e(f"s_cbranch_scc1 {skip}")
+        self.e(f"s_cmp_lg_u32 {self.sr('Wave')}, 0")
+        self.e(f"s_cbranch_scc1 {skip}")
+        self.e(f"s_cmp_ge_u32 {self.sr('Begin')}, 62")
+        self.e(f"s_cbranch_scc1 {skip}")
+        self.e(f"s_memrealtime {s(self.S['T'] + 4, 2)}")
+        self.e(f"s_lshl_b32 {t(0)}, {self.sr('L')}, 9")          # 64 x 8 bytes per workgroup
+        self.e(f"s_add_u32 {t(2)}, {s(tl)}, {t(0)}")
+        self.e(f"s_addc_u32 {t(3)}, {s(tl + 1)}, 0")
+        self.e(f"s_lshl_b32 {t(0)}, {self.sr('Begin')}, 3")
+        self.e(f"s_add_u32 {self.sr('Begin')}, {self.sr('Begin')}, 1")
+        self.e("s_waitcnt lgkmcnt(0)")
+        self.e("s_mov_b64 exec, 1")
+        self.e(f"v_mov_b32 {self.vr('Tmp', 0)}, {t(0)}")           # byte offset of the new stamp - 16
+        self.e(f"v_mov_b32 {self.vr('Tmp', 1)}, {t(4)}")
+        self.e(f"global_store_dword {self.vr('Tmp', 0)}, {self.vr('Tmp', 1)}, {s(self.S['T'] + 2, 2)} offset:16")
+        self.e(f"v_mov_b32 {self.vr('Tmp', 1)}, {t(5)}")
+        self.e(f"global_store_dword {self.vr('Tmp', 0)}, {self.vr('Tmp', 1)}, {s(self.S['T'] + 2, 2)} offset:20")
+        self.e(f"v_mov_b32 {self.vr('Tmp', 1)}, {self.sr('Begin')}")
+        self.e(f"global_store_dword {self.vr('Zero')}, {self.vr('Tmp', 1)}, {s(self.S['T'] + 2, 2)}")
+        self.e("s_mov_b64 exec, -1")
+        self.label(skip)
+
     # ------------------------------------------------------------------ whole kernel
     def body(self):
         S, t = self.S, self.t
@@ -622,6 +656,7 @@ class Kernel:
         e(f"s_load_dwordx8 {s(8, 8)}, s[0:1], 0x0")
         e(f"s_load_dwordx16 {s(16, 16)}, s[0:1], 0x20")
         e(f"s_load_dwordx8 {s(32, 8)}, s[0:1], 0x60")
+        e(f"s_load_dwordx2 {s(40, 2)}, s[0:1], 0x80")
         e(f"v_and_b32 {self.vr('Tmp', 1)}, 0x3ff, v0")
         e(f"v_lshrrev_b32 {self.vr('Tmp')}, 6, {self.vr('Tmp', 1)}")
         e(f"v_and_b32 {self.vr('Lane')}, 63, {self.vr('Tmp', 1)}")
@@ -694,6 +729,8 @@ class Kernel:
         e(f"s_lshl_b32 {t(0)}, {self.sr('KwSpw')}, 12")
         e(f"v_add_u32 {self.vr('LdsWr')}, {t(0)}, {tmp(0)}")
 
+        e(f"s_mov_b32 {self.sr('Begin')}, 0")  # from here on: number of timeline stamps
+        self.stamp()
         # ---- prologue: unit 0 -> buffer 0 with the patches of unit 1 already in flight.  Unit 0's
         # patches land in registers that are free until the first chunk (MPX, VB), so that both
         # units' loads leave together and the kernel pays one trip to memory, not two.
@@ -726,6 +763,7 @@ class Kernel:
 
         seg_loop, regular, check, done = (self.newlabel(x) for x in ("seg", "regular", "check", "done"))
         plain_seg, epi_plain, after_epi = (self.newlabel(x) for x in ("plainseg", "epiplain", "afterepi"))
+        self.stamp()
         self.label(seg_loop)
         # this segment: chunks Cm .. SegEnd-1 of tile Tm.  Kind: 1 publish (starts inside the tile),
         # 2 merge (ends inside the tile), 0 whole tile.
@@ -751,6 +789,7 @@ class Kernel:
         e(f"s_cmp_lt_u32 {self.sr('Cm')}, {self.sr('SegEnd')}")
         e(f"s_cbranch_scc1 {regular}")
         self.label(epi_plain)
+        self.stamp()
         pub = self.newlabel("publish")
         e(f"s_cmp_eq_u32 {self.sr('Kind')}, 1")
         e(f"s_cbranch_scc1 {pub}")
@@ -763,6 +802,7 @@ class Kernel:
         self.store_flag(self.vr("One"))
         e("s_waitcnt vmcnt(0)")
         self.label(after_epi)
+        self.stamp()
         e(f"s_cmp_lt_u32 {self.sr('G')}, {self.sr('Nunits')}")
         e(f"s_cbranch_scc0 {done}")
         e(f"s_add_u32 {self.sr('Tm')}, {self.sr('Tm')}, 1")
@@ -785,7 +825,7 @@ class Kernel:
 \t.amdhsa_kernel {n}
 \t\t.amdhsa_group_segment_fixed_size 0
 \t\t.amdhsa_private_segment_fixed_size 0
-\t\t.amdhsa_kernarg_size 128
+\t\t.amdhsa_kernarg_size 136
 \t\t.amdhsa_user_sgpr_count 2
 \t\t.amdhsa_user_sgpr_kernarg_segment_ptr 1
 \t\t.amdhsa_system_sgpr_workgroup_id_x 1
@@ -809,12 +849,17 @@ class Kernel:
         args += "\n" + "\n".join(f"""      - .offset:         {32 + 4 * i}
         .size:           4
         .value_kind:     by_value""" for i in range(24))
+        args += """
+      - .address_space:  global
+        .offset:         128
+        .size:           8
+        .value_kind:     global_buffer"""
         return f"""  - .agpr_count:     256
     .args:
 {args}
     .group_segment_fixed_size: 0
     .kernarg_segment_align: 8
-    .kernarg_segment_size: 128
+    .kernarg_segment_size: 136
     .max_flat_workgroup_size: 256
     .name:           {self.name}
     .private_segment_fixed_size: 0

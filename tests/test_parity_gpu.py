@@ -615,5 +615,32 @@ def test_call_replays_from_a_captured_graph(ocn, oracle, torch_gpu, N, C, H, K):
         ocn.set_stream(None)
 
 
+def test_timeline_buffer_records_monotone_stamps(ocn, oracle, torch_gpu):
+    # bench support of the assembly kernels: every workgroup's first wave records the realtime
+    # counter at its start, after its prologue and around every output transform; recording must
+    # not change the result, and stops when the buffer is taken away
+    print("timeline", flush=True)
+    torch = torch_gpu
+    N, C, H, K = 64, 16, 40, 128  # 800 workgroup tiles on a persistent grid: several tiles per workgroup
+    x, w = make_tensors(ocn, N, C, H, H, K)
+    r = Runner(ocn, torch, x, w)
+    y_plain = r.split()
+    buf = torch.zeros(1024 * 64, dtype=torch.int64, device="cuda")
+    try:
+        ocn.set_timeline_buffer(buf)
+        y_rec = r.split()
+    finally:
+        ocn.set_timeline_buffer(None)
+    assert np.array_equal(y_plain, y_rec)
+    rec = buf.cpu().numpy().reshape(-1, 64)
+    nwg = int((rec[:, 0] > 0).sum())
+    assert nwg >= 8 and (rec[:nwg, 0] >= 4).all() and (rec[:nwg, 0] % 2 == 0).all()
+    for v in ocn.read_timeline(buf, nwg):
+        assert all(b >= a for a, b in zip(v, v[1:])) and 0 <= v[0] and v[-1] < 1e4
+    buf.zero_()
+    r.split()
+    assert int(buf.abs().sum()) == 0
+
+
 def test_init_accepts_this_device(ocn, torch_gpu):
     ocn.init()
