@@ -86,7 +86,19 @@ class Layer:
                                      self.H, self.K, warmup=warmup, iters=iters)
 
 
-def miopen_column(torch, lay, warmup=10, iters=50):
+def settle(torch, lay, ms):
+    """Untimed: run the step back to back for `ms` of wall time.  After an idle period (tensor
+    set-up, the CPU leg) the device needs some tens of milliseconds of continuous work before
+    its clocks and its launch path are in their sustained state; a layer of a network runs in
+    that state, so every timed region here starts from it."""
+    t_end = time.perf_counter() + ms * 1e-3
+    while time.perf_counter() < t_end:
+        for _ in range(200):
+            lay.step()
+        torch.cuda.synchronize()
+
+
+def miopen_column(torch, lay, warmup=10, iters=200, settle_ms=150.0):
     """Informational only, never an oracle: ms per call of torch.nn.functional.conv2d (MIOpen's
     own choice of fp32 algorithm) on the same layer in NCHW / KCRS, the analogue of the
     reference bench's cuDNN column (src/openCNN_winograd.cu:449-464)."""
@@ -95,8 +107,13 @@ def miopen_column(torch, lay, warmup=10, iters=50):
     torch.backends.cudnn.benchmark = True  # let MIOpen search instead of taking its first guess
     for _ in range(warmup):
         y = torch.nn.functional.conv2d(x, w, padding=1)
-    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
     torch.cuda.synchronize()
+    t_end = time.perf_counter() + settle_ms * 1e-3  # same sustained state as the library's column
+    while time.perf_counter() < t_end:
+        for _ in range(100):
+            y = torch.nn.functional.conv2d(x, w, padding=1)
+        torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
     ev[0].record()
     for _ in range(iters):
         y = torch.nn.functional.conv2d(x, w, padding=1)
@@ -175,6 +192,8 @@ def main():
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(FP32_LAYERS))
+    ap.add_argument("--settle-ms", type=float, default=300.0,
+                    help="untimed back-to-back run before every measurement (0: measure from idle)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-layers", action="store_true", help="skip the per-layer table")
     ap.add_argument("--timeline", action="store_true",
@@ -199,6 +218,7 @@ def main():
     layer = Layer(ocn, torch, args.workload)
     fd, fm, bmin = work(layer.N, layer.C, layer.H, layer.K)
 
+    settle(torch, layer, args.settle_ms)
     for _ in range(args.warmup):
         layer.step()
     torch.cuda.synchronize()
@@ -222,6 +242,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settle_ms": args.settle_ms,
         "ms_per_step": ms_step,
         "higher_is_better": True,
         "scaling": "weak",
@@ -271,12 +292,13 @@ def main():
             for label, prec, peak in precisions:
                 try:
                     ocn.set_operand_precision(prec)
+                    settle(torch, lay, args.settle_ms / 2)
                     tot, mn, fx = lay.kernel_times(20, 200)
                 finally:
                     ocn.set_operand_precision(ocn.F32)
                 extra = {}
                 if args.miopen and label == "f32":
-                    extra["ms_miopen_conv2d_fp32"] = miopen_column(torch, lay)
+                    extra["ms_miopen_conv2d_fp32"] = miopen_column(torch, lay, settle_ms=args.settle_ms / 2)
                 rows.append({
                     **extra,
                     "workload": name, "gemm_operands": label, "ms_per_layer": tot, "ms_fused_kernel": mn,
