@@ -44,10 +44,12 @@ thread_local const char* t_last_error = "";
 
 // ---- hand-scheduled assembly kernels (gen_wino_f32_asm.py), loaded from the embedded code object
 extern "C" const char opencnn_wino_f32_asm_hsaco[];
+extern "C" const char opencnn_wino_h16_asm_hsaco[];  // gen_wino_h16_asm.py
 
 struct AsmKernels {
-  hipModule_t module = nullptr;
+  hipModule_t module = nullptr, module_h16 = nullptr;
   hipFunction_t kw2 = nullptr, kw4 = nullptr, kw2_ragged = nullptr, kw4_ragged = nullptr;
+  hipFunction_t f16_kw4 = nullptr, bf16_kw4 = nullptr;
   unsigned* split_sync = nullptr;  // device address of g_split_sync on this device
   bool ready = false;
 };
@@ -68,6 +70,9 @@ int asm_kernels(const AsmKernels** out) {
     if ((e = hipModuleGetFunction(&k.kw4, k.module, "wino_f32_asm_kw4")) != hipSuccess) return (int)e;
     if ((e = hipModuleGetFunction(&k.kw2_ragged, k.module, "wino_f32_asm_kw2_ragged")) != hipSuccess) return (int)e;
     if ((e = hipModuleGetFunction(&k.kw4_ragged, k.module, "wino_f32_asm_kw4_ragged")) != hipSuccess) return (int)e;
+    if ((e = hipModuleLoadData(&k.module_h16, opencnn_wino_h16_asm_hsaco)) != hipSuccess) return (int)e;
+    if ((e = hipModuleGetFunction(&k.f16_kw4, k.module_h16, "wino_f16_asm_kw4")) != hipSuccess) return (int)e;
+    if ((e = hipModuleGetFunction(&k.bf16_kw4, k.module_h16, "wino_bf16_asm_kw4")) != hipSuccess) return (int)e;
     if ((e = hipGetSymbolAddress(reinterpret_cast<void**>(&k.split_sync), HIP_SYMBOL(opencnn::g_split_sync))) != hipSuccess)
       return (int)e;
     // 64 KB of dynamic LDS for KW = 2 is the default limit exactly; nothing to raise
@@ -224,9 +229,8 @@ int launch_h16(opencnn::ConvArgs a, int precision, hipStream_t st) {
 // Grid of the hand-scheduled kernels for this layer, or 0 when they do not take it.  One
 // persistent launch whose workgroups share the (tile, chunk) units evenly; it needs whole filter
 // blocks (kw > 1) and at least one tile per workgroup (a tile then has at most two contributors).
-int asm_grid(const opencnn::ConvArgs& a, int kw, int* grid) {
+int asm_grid(const opencnn::ConvArgs& a, int kw, int chunks, int* grid) {
   *grid = 0;
-  const int chunks = (a.C + 7) / 8;
   if (kw == 1 || (long long)a.nblocks * chunks > kMaxElems) return 0;
   // per-lane store offsets: four filter rows plus one image row and column, in bytes
   if (((long long)a.N * a.H * a.W * 4 + (long long)(a.W + 1) * a.N) * 4 > kMaxElems) return 0;
@@ -240,11 +244,14 @@ int asm_grid(const opencnn::ConvArgs& a, int kw, int* grid) {
   return 0;
 }
 
-int launch_asm(const opencnn::ConvArgs& a, int kw, int grid, bool ragged, size_t lds_bytes,
-               hipStream_t st) {
-  const AsmKernels* ak = nullptr;
-  if (int e = asm_kernels(&ak)) return e;
-  const int chunks = (a.C + 7) / 8;
+// chunks: units per workgroup tile; usw_bytes: size of the transformed filter; tile_split: the
+// divisor that takes a workgroup tile index apart (fp32: column blocks, filter-block major
+// order; fp16 / bf16: filter blocks, column-block major order).
+// lockstep_log2 >= 0 (fp16 / bf16 kernels only): one line of units per filter block, 2^lockstep_log2
+// filter blocks; tile_split is then their number and c_real (the mode flag of those kernels) 0.
+int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmKernels* ak, hipFunction_t fn, int chunks,
+                      long long usw_bytes, int tile_split, int c_real, int lockstep_log2, int grid,
+                      size_t lds_bytes, hipStream_t st) {
   AsmKernArgs ka{};
   ka.x = a.x;
   ka.usw = a.usw;
@@ -257,28 +264,74 @@ int launch_asm(const opencnn::ConvArgs& a, int kw, int grid, bool ragged, size_t
   ka.tiles_w = a.tiles_w;
   ka.ngroups = a.ngroups;
   ka.colgroups = a.colgroups;
-  ka.colblocks = a.colblocks;
+  ka.colblocks = tile_split;
   ka.Q = chunks * 2;
   ka.HWN4 = a.N * a.H * a.W * 4;
-  ka.c_real = a.C;
+  ka.c_real = c_real;
   ka.k_real = a.K;
-  const long long total = (long long)a.nblocks * chunks;
-  ka.units_q = (int32_t)(total / grid);
-  ka.units_rem = (int32_t)(total % grid);
-  ka.usw_bytes = (int32_t)(padded_c(a.C) * 16 * padded_k(a.K) * 4);
+  long long total = (long long)a.nblocks * chunks;
+  int ranges = grid;
+  if (lockstep_log2 >= 0) {
+    total >>= lockstep_log2;
+    ranges >>= lockstep_log2;
+  }
+  ka.units_q = (int32_t)(total / ranges);
+  ka.units_rem = (int32_t)(total % ranges);
+  ka.usw_bytes = (int32_t)usw_bytes;
   ka.grid_per_xcd = grid % 8 == 0 ? grid / 8 : 0;  // 0: no XCD-aware block order
   ka.timeline = (size_t)grid * 64 * sizeof(long long) <= g_timeline_bytes.load() ? g_timeline.load() : nullptr;
   magic_divisor((uint32_t)chunks, &ka.m_chunks, &ka.s_chunks);
-  magic_divisor((uint32_t)a.colblocks, &ka.m_colblocks, &ka.s_colblocks);
+  magic_divisor((uint32_t)tile_split, &ka.m_colblocks, &ka.s_colblocks);
+  if (lockstep_log2 >= 0) ka.s_colblocks = (uint32_t)lockstep_log2;
   magic_divisor((uint32_t)a.ngroups, &ka.m_ngroups, &ka.s_ngroups);
   magic_divisor((uint32_t)a.tiles_w, &ka.m_tiles_w, &ka.s_tiles_w);
   size_t ka_size = sizeof(ka);
   void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &ka, HIP_LAUNCH_PARAM_BUFFER_SIZE, &ka_size,
                    HIP_LAUNCH_PARAM_END};
-  const hipFunction_t fn =
-      ragged ? (kw == 4 ? ak->kw4_ragged : ak->kw2_ragged) : (kw == 4 ? ak->kw4 : ak->kw2);
   return (int)hipModuleLaunchKernel(fn, (unsigned)grid, 1, 1, 256, 1, 1, (unsigned)lds_bytes, st,
                                     nullptr, extra);
+}
+
+int launch_asm(const opencnn::ConvArgs& a, int kw, int grid, bool ragged, size_t lds_bytes,
+               hipStream_t st) {
+  const AsmKernels* ak = nullptr;
+  if (int e = asm_kernels(&ak)) return e;
+  const hipFunction_t fn =
+      ragged ? (kw == 4 ? ak->kw4_ragged : ak->kw2_ragged) : (kw == 4 ? ak->kw4 : ak->kw2);
+  return launch_asm_kernel(a, ak, fn, (a.C + 7) / 8, padded_c(a.C) * 16 * padded_k(a.K) * 4, a.colblocks,
+                           a.C, -1, grid, lds_bytes, st);
+}
+
+// The hand-scheduled fp16 / bf16 kernels (gen_wino_h16_asm.py) take whole 128-filter blocks and
+// 16-channel chunks of shapes inside the reference's tiling; *launched stays false otherwise.
+int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* launched) {
+  *launched = false;
+  if (a.N % 32 != 0 || a.C % 16 != 0 || a.K % 128 != 0) return 0;
+  if ((long long)a.N * a.H * a.W * 4 * 4 > kMaxElems) return 0;  // four-channel slab in bytes
+  const int kblocks = a.kgroups / 4, chunks = a.C / 16;
+  const long long nblocks = (long long)a.colgroups * kblocks;
+  if (nblocks > kMaxElems / 8) return 0;
+  a.nblocks = (int)nblocks;
+  a.colblocks = a.colgroups;
+  int grid = 0;
+  if (int e = asm_grid(a, 4, chunks, &grid)) return e;
+  if (grid == 0) return 0;
+  const AsmKernels* ak = nullptr;
+  if (int e = asm_kernels(&ak)) return e;
+  const hipFunction_t fn = precision == OPENCNN_BF16 ? ak->bf16_kw4 : ak->f16_kw4;
+  const size_t lds_bytes = 2 * 16 * 2 * 4 * 32 * sizeof(unsigned);  // two buffers of V
+  // How the units are dealt.  While the whole 2-byte transformed filter leaves room in an XCD's
+  // 4 MB L2 and the filter blocks are a power of two that divides the grid: one line of units per
+  // filter block, walked in lockstep by neighbouring workgroups (the patches the filter blocks
+  // share are read from HBM once).  Else one filter-block-major line as in the fp32 kernels.
+  const long long usw_bytes = (long long)a.C * 16 * a.K * 2;
+  int log2k = 0;
+  while ((1 << log2k) < kblocks) ++log2k;
+  const bool lockstep = usw_bytes <= (2 << 20) && (1 << log2k) == kblocks && grid % kblocks == 0;
+  const int e = lockstep ? launch_asm_kernel(a, ak, fn, chunks, usw_bytes, kblocks, 0, log2k, grid, lds_bytes, st)
+                         : launch_asm_kernel(a, ak, fn, chunks, usw_bytes, a.colblocks, 1, -1, grid, lds_bytes, st);
+  *launched = e == 0;
+  return e;
 }
 
 // The HIP C++ kernels: register variant (kw == 1), LDS variant, and the LDS variant as one
@@ -350,7 +403,16 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   a.kgroups = (filt_k + 31) / 32;
   a.nblocks = a.colblocks = 0;
   const int precision = g_precision.load();
-  if (precision != OPENCNN_F32) return launch_h16(a, precision, st);
+  if (precision != OPENCNN_F32) {
+    const int v = g_variant.load();
+    if (v == OPENCNN_KERNEL_ASM || v == OPENCNN_KERNEL_AUTO) {
+      bool launched = false;
+      if (int e = launch_h16_asm(a, precision, st, &launched)) return e;
+      if (launched) return 0;
+      REQUIRE(v != OPENCNN_KERNEL_ASM);
+    }
+    return launch_h16(a, precision, st);
+  }
 
   // Waves per workgroup that share one column tile (and split its input transform): as many as
   // the (rounded-up) filter groups fill whole workgroups of.
@@ -369,7 +431,7 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
 
   if (variant == OPENCNN_KERNEL_ASM || variant == OPENCNN_KERNEL_AUTO) {
     int grid = 0;
-    if (int e = asm_grid(a, kw, &grid)) return e;
+    if (int e = asm_grid(a, kw, (a.C + 7) / 8, &grid)) return e;
     if (grid > 0) return launch_asm(a, kw, grid, ragged, lds_bytes, st);
     REQUIRE(variant != OPENCNN_KERNEL_ASM);
   }

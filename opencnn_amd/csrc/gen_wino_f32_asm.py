@@ -116,6 +116,10 @@ class Kernel:
 
     # ------------------------------------------------------------------ registers
     def alloc(self):
+        self.alloc_sgprs()
+        self.alloc_vgprs()
+
+    def alloc_sgprs(self):
         # s[0:1] kernel argument pointer, s2 workgroup id, s[8:15] the four pointers,
         # s[16:39] the 24 ints, s[40:41] the timeline pointer, s42.. everything else
         S = Alloc(42, 102)
@@ -136,6 +140,7 @@ class Kernel:
         self.S["T"] = S.get("T", 8, 2)  # temporaries T0..T7 (T6:T7 = division pair)
         self.sgpr_count = S.next
 
+    def alloc_vgprs(self):
         V = Alloc(1, 256)
         self.V = {}
         for n, cnt, al in [("Lane", 1, 1), ("LaneX", 1, 1), ("Lane8", 1, 1), ("Lane8b", 1, 1),
@@ -170,12 +175,21 @@ class Kernel:
         self.e(f"s_lshr_b64 {s(t6, 2)}, {s(t6, 2)}, {sh}")
         self.e(f"s_mov_b32 {dst}, {s(t6)}")
 
-    def decode(self, T):
-        """Workgroup tile T -> Dkb (filter block), Dlive, Dng, Dty, Dtx of this wave's column tile."""
+    def split_tile(self, T):
+        """Workgroup tile T -> Dkb (filter block) and T0 (column block): filter-block major."""
         t = self.t
         self.div(self.sr("Dkb"), T, self.sr("Mcb"), self.sr("Scb"))
         self.e(f"s_mul_i32 {t(0)}, {self.sr('Dkb')}, {self.sr('Colblocks')}")
         self.e(f"s_sub_u32 {t(0)}, {T}, {t(0)}")  # column block
+
+    def filter_block(self, dst, T):
+        """dst = filter block of workgroup tile T (may use T0, T1)."""
+        self.div(dst, T, self.sr("Mcb"), self.sr("Scb"))
+
+    def decode(self, T):
+        """Workgroup tile T -> Dkb (filter block), Dlive, Dng, Dty, Dtx of this wave's column tile."""
+        t = self.t
+        self.split_tile(T)
         if self.CW == 2:
             self.e(f"s_lshl_b32 {t(0)}, {t(0)}, 1")
             self.e(f"s_add_u32 {t(0)}, {t(0)}, {self.sr('Cw')}")
@@ -403,12 +417,12 @@ class Kernel:
             self.read_v("VA", 0, p)
 
     # ------------------------------------------------------------------ cursors
-    def advance_p(self):
-        """P cursor -> unit G+2 when there is one.  The common case (same tile) falls through
+    def advance_p(self, ahead=2):
+        """P cursor -> unit G+ahead when there is one.  The common case (same tile) falls through
         without a taken branch; the tile switch lives out of line, behind the kernel's end."""
         rare, back = self.newlabel("p_switch"), self.newlabel("p_back")
         t = self.t
-        self.e(f"s_add_u32 {t(0)}, {self.sr('G')}, 2")
+        self.e(f"s_add_u32 {t(0)}, {self.sr('G')}, {ahead}")
         self.e(f"s_cmp_lt_u32 {t(0)}, {self.sr('Nunits')}")
         self.e(f"s_addc_u32 {self.sr('Cp')}, {self.sr('Cp')}, 0")  # + SCC
         self.e(f"s_cmp_eq_u32 {self.sr('Cp')}, {self.sr('Chunks')}")
@@ -437,7 +451,7 @@ class Kernel:
         self.label(rare)
         self.e(f"s_mov_b32 {self.sr('Cq')}, 0")
         self.e(f"s_add_u32 {self.sr('Tq')}, {self.sr('Tq')}, 1")
-        self.div(t(0), self.sr("Tq"), self.sr("Mcb"), self.sr("Scb"))
+        self.filter_block(t(0), self.sr("Tq"))
         self.e(f"s_lshl_b32 {t(0)}, {t(0)}, {self.KW.bit_length() - 1}")
         self.e(f"s_add_u32 {self.sr('KgQ')}, {t(0)}, {self.sr('Kw')}")
         self.e(f"s_branch {back}")
@@ -650,6 +664,21 @@ class Kernel:
 
     # ------------------------------------------------------------------ whole kernel
     def body(self):
+        self.head()
+        self.lane_setup()
+        self.e(f"s_mov_b32 {self.sr('Begin')}, 0")  # from here on: number of timeline stamps
+        self.stamp()
+        self.prologue()
+        self.segments()
+
+    SLAB_CHANNELS = 2  # channels behind one patch-load descriptor
+
+    def range_owner(self):
+        """The register that numbers this workgroup's range of units."""
+        return self.sr("L")
+
+    def head(self):
+        """Kernel arguments, wave / workgroup identity, the unit range, cursors, descriptors."""
         S, t = self.S, self.t
         e = self.e
         KWLOG = self.KW.bit_length() - 1
@@ -680,10 +709,11 @@ class Kernel:
         e(f"s_cmp_eq_u32 {self.sr('GridPerXcd')}, 0")
         e(f"s_cselect_b32 {self.sr('L')}, s2, {t(0)}")
         # units [Begin, Begin + Nunits): the first UnitsRem blocks take one more
-        e(f"s_mul_i32 {self.sr('Begin')}, {self.sr('L')}, {self.sr('UnitsQ')}")
-        e(f"s_min_u32 {t(0)}, {self.sr('L')}, {self.sr('UnitsRem')}")
+        owner = self.range_owner()
+        e(f"s_mul_i32 {self.sr('Begin')}, {owner}, {self.sr('UnitsQ')}")
+        e(f"s_min_u32 {t(0)}, {owner}, {self.sr('UnitsRem')}")
         e(f"s_add_u32 {self.sr('Begin')}, {self.sr('Begin')}, {t(0)}")
-        e(f"s_cmp_lt_u32 {self.sr('L')}, {self.sr('UnitsRem')}")
+        e(f"s_cmp_lt_u32 {owner}, {self.sr('UnitsRem')}")
         e(f"s_cselect_b32 {t(0)}, 1, 0")
         e(f"s_add_u32 {self.sr('Nunits')}, {self.sr('UnitsQ')}, {t(0)}")
         self.div(self.sr("Tm"), self.sr("Begin"), self.sr("Mch"), self.sr("Sch"))
@@ -695,7 +725,7 @@ class Kernel:
             e(f"s_mov_b32 {self.sr(n)}, {self.sr('Cm')}")
         e(f"s_lshl_b32 {self.sr('ColStep')}, {self.sr('N')}, 2")
         e(f"s_mul_i32 {self.sr('RowStep')}, {self.sr('ColStep')}, {self.sr('W')}")
-        e(f"s_lshl_b32 {self.sr('Slab')}, {self.sr('HWN4')}, 1")
+        e(f"s_lshl_b32 {self.sr('Slab')}, {self.sr('HWN4')}, {self.SLAB_CHANNELS.bit_length() - 1}")
         # descriptors: words 2 (num_records) and 3 (flags) never change
         e(f"s_mov_b32 {s(S['RsrcX'] + 2)}, {self.sr('Slab')}")
         e(f"s_mov_b32 {s(S['RsrcX'] + 3)}, 0x{FLAGS:x}")
@@ -705,7 +735,10 @@ class Kernel:
         e(f"s_mov_b32 {s(S['RsrcU'] + 3)}, 0x{FLAGS:x}")
         e(f"s_mov_b32 {s(S['RsrcY'] + 2)}, 0x{OOB:x}")
         e(f"s_mov_b32 {s(S['RsrcY'] + 3)}, 0x{FLAGS:x}")
-        # per lane
+
+    def lane_setup(self):
+        """Per-lane registers: patch / store offsets, filter-load offsets, LDS addresses."""
+        t, e = self.t, self.e
         tmp = lambda i: self.vr("Tmp", i)
         e(f"v_lshrrev_b32 {tmp(0)}, 5, {self.vr('Lane')}")             # hsel
         e(f"v_and_b32 {tmp(1)}, 31, {self.vr('Lane')}")                # nl
@@ -729,11 +762,11 @@ class Kernel:
         e(f"s_lshl_b32 {t(0)}, {self.sr('KwSpw')}, 12")
         e(f"v_add_u32 {self.vr('LdsWr')}, {t(0)}, {tmp(0)}")
 
-        e(f"s_mov_b32 {self.sr('Begin')}, 0")  # from here on: number of timeline stamps
-        self.stamp()
-        # ---- prologue: unit 0 -> buffer 0 with the patches of unit 1 already in flight.  Unit 0's
-        # patches land in registers that are free until the first chunk (MPX, VB), so that both
-        # units' loads leave together and the kernel pays one trip to memory, not two.
+    def prologue(self):
+        """Unit 0 -> buffer 0 with the patches of unit 1 already in flight.  Unit 0's patches land
+        in registers that are free until the first chunk (MPX, VB), so that both units' loads
+        leave together and the kernel pays one trip to memory, not two."""
+        e = self.e
         self.decode(self.sr("Tm"))
         self.m_tile_setup()
         e(f"s_mov_b32 {self.sr('KgQ')}, {self.sr('KgM')}")
@@ -761,6 +794,10 @@ class Kernel:
         self.end_of_chunk()
         e("s_waitcnt vmcnt(0)")  # the first chunk counts on a queue without surprises
 
+    def segments(self):
+        """The segment loop: chunks of one tile, then its output transform (plain, published, or
+        started from a published partial tile)."""
+        t, e = self.t, self.e
         seg_loop, regular, check, done = (self.newlabel(x) for x in ("seg", "regular", "check", "done"))
         plain_seg, epi_plain, after_epi = (self.newlabel(x) for x in ("plainseg", "epiplain", "afterepi"))
         self.stamp()

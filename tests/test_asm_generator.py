@@ -73,3 +73,71 @@ def test_output_assembles_for_gfx950(tmp_path):
     assert obj.stat().st_size > 10000
     lld = shutil.which("ld.lld") or "/opt/rocm/lib/llvm/bin/ld.lld"
     subprocess.run([lld, "-shared", str(obj), "-o", str(tmp_path / "k.hsaco")], check=True)
+
+
+# ---------------------------------------------------------------- fp16 / bf16 kernels
+GEN_H16 = os.path.join(ROOT, "opencnn_amd", "csrc", "gen_wino_h16_asm.py")
+
+
+@pytest.fixture(scope="module")
+def gen_h16(gen):
+    import sys
+    sys.modules.setdefault("gen_wino_f32_asm", gen)  # the fp16 / bf16 generator extends its Kernel class
+    spec = importlib.util.spec_from_file_location("gen_wino_h16_asm", GEN_H16)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_h16_register_budget(gen_h16, bf16):
+    k = gen_h16.KernelH16(bf16)
+    assert k.vgpr_count <= 256
+    assert k.sgpr_count <= 98
+    assert len(set(k.MP)) == 64
+    live_at_boundary = set()
+    for name, n in (("U", 64), ("DA0", 16), ("DB0", 16), ("DA1", 16), ("DB1", 16), ("VOFF", 16),
+                    ("Off", 4), ("Eff", 4), ("Lane16", 4)):
+        live_at_boundary |= set(range(k.V[name], k.V[name] + n))
+    assert not live_at_boundary & set(k.MP), "partial tile would land on live pipeline registers"
+    # MFMA operand tuples start on even registers
+    assert k.V["U"] % 2 == 0 and k.V["VR"] % 2 == 0
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_h16_kernel_text_invariants(gen_h16, bf16):
+    k = gen_h16.KernelH16(bf16)
+    k.body()
+    text = "\n".join(k.lines)
+    op = "v_mfma_f32_32x32x16_bf16" if bf16 else "v_mfma_f32_32x32x16_f16"
+    other = "v_mfma_f32_32x32x16_f16" if bf16 else "v_mfma_f32_32x32x16_bf16"
+    # six chunk bodies (plain first / merging first / steady state, each for even and odd units)
+    assert text.count(op) == 6 * 16 and other not in text
+    assert text.count("s_barrier") == 6 + 1
+    # first chunk of a tile: 16 MFMAs from the constant 0; a merging segment keeps four accumulators
+    assert len(re.findall(op + r" [^\n]*, 0$", text, re.M)) == 2 * 16 + 2 * 12
+    cvt = "v_cvt_pk_bf16_f32" if bf16 else "v_cvt_pk_f16_f32"
+    assert text.count(cvt) == 7 * 16
+    # per chunk body: 16 filter loads, 32 patch loads; prologue: 16 + 3 * 32
+    assert text.count("buffer_load_dwordx4") == 7 * 16
+    assert len(re.findall(r"buffer_load_dword v", text)) == 6 * 32 + 3 * 32 + 64  # + the merge's 64
+    assert len(re.findall(r"buffer_store_dword", text)) == 2 * 64
+    assert all(int(n) <= 63 for n in re.findall(r"vmcnt\((\d+)\)", text))
+    assert all(int(n) <= 15 for n in re.findall(r"lgkmcnt\((\d+)\)", text))
+    labels = re.findall(r"^(\.L\w+):", text, re.M)
+    assert len(labels) == len(set(labels))
+    for target in re.findall(r"s_c?branch\w* (\.L\w+)", text):
+        assert target in labels
+    # LDS: two 16 KB buffers; every access stays below 32 KB for the largest lane offsets
+    assert max(int(n) for n in re.findall(r"offset1:(\d+)", text)) * 256 + 0x4000 + 0x80 + 636 < 32768
+
+
+@pytest.mark.skipif(not os.path.exists(CLANG), reason="ROCm LLVM assembler not installed")
+def test_h16_output_assembles_for_gfx950(tmp_path):
+    src = tmp_path / "k.s"
+    with open(src, "w") as f:
+        subprocess.run(["python3", GEN_H16], check=True, stdout=f)
+    obj = tmp_path / "k.o"
+    subprocess.run([CLANG, "-x", "assembler", "-target", "amdgcn-amd-amdhsa", "-mcpu=gfx950",
+                    "-c", str(src), "-o", str(obj)], check=True)
+    assert obj.stat().st_size > 10000

@@ -498,6 +498,60 @@ def test_reduced_precision_operands(ocn, oracle, torch_gpu, prec, N, C, H, K, xr
     print(f"  rel-L2 vs quantised restatement {rel:.2e}, vs fp64 direct {rel64:.2e}", flush=True)
 
 
+# (N, C, H, W, K) for the hand-scheduled fp16 / bf16 kernels (K % 128 == 0, C % 16 == 0):
+# the benchmark configuration (two filter blocks in lockstep); one tile per workgroup; one
+# 16-channel chunk; three filter blocks and an 8 MB transformed filter (one filter-block-major
+# line of units); tiles cut between workgroups with one, two and four filter blocks; odd sizes
+H16_ASM_SHAPES = [(128, 256, 14, 14, 256), (32, 32, 6, 6, 128), (32, 16, 9, 9, 256), (64, 48, 9, 9, 384),
+                  (32, 512, 5, 5, 512), (64, 32, 40, 40, 128), (64, 64, 21, 21, 256), (32, 32, 30, 30, 512),
+                  (32, 32, 31, 9, 128), (96, 48, 1, 1, 128)]
+
+
+@pytest.mark.parametrize("prec", ["f16", "bf16"])
+@pytest.mark.parametrize("N,C,H,W,K", H16_ASM_SHAPES)
+def test_reduced_precision_assembly_kernels(ocn, oracle, torch_gpu, prec, N, C, H, W, K):
+    # selected explicitly (an unsupported shape would raise, not fall back); against the
+    # quantised restatement, the fp64 direct convolution, a second call, and the HIP C++ kernel
+    print(f"reduced asm {prec} N={N} C={C} H={H} W={W} K={K}", flush=True)
+    x, w = make_tensors(ocn, N, C, H, W, K)
+    r = Runner(ocn, torch_gpu, x, w)
+    try:
+        ocn.set_operand_precision(ocn.F16 if prec == "f16" else ocn.BF16)
+        ocn.set_kernel_variant(ocn.KERNEL_ASM)
+        y = r.split()
+        y2 = r.split()
+        ocn.set_kernel_variant(ocn.KERNEL_HIP)
+        y_hip = r.split()
+    finally:
+        ocn.set_kernel_variant(ocn.KERNEL_AUTO)
+        ocn.set_operand_precision(ocn.F32)
+    assert not np.isnan(y).any(), "an output element was never written"
+    assert np.array_equal(y, y2)
+    rel64, _, _ = oracle.compare(y, oracle.direct_conv_f64(x, w))
+    assert rel64 <= REL_L2_DIRECT_REDUCED[prec], f"rel-L2 vs fp64 direct {rel64:.3e}"
+    # same operands, same roundings; only the order of the fp32 sums inside the MFMA chain differs
+    rel_hip, _, _ = oracle.compare(y, y_hip)
+    assert rel_hip <= REL_L2_QUANTISED_RESTATEMENT, f"rel-L2 vs the HIP kernel {rel_hip:.3e}"
+    if H == W:
+        rel, _, _ = oracle.compare(y, oracle.winograd_f32(x, w, 1 if prec == "f16" else 2))
+        assert rel <= REL_L2_QUANTISED_RESTATEMENT, f"rel-L2 vs quantised restatement {rel:.3e}"
+
+
+def test_reduced_precision_assembly_variant_rejects_other_shapes(ocn, torch_gpu):
+    x, w = make_tensors(ocn, 32, 16, 6, 6, 64)  # K % 128 != 0: the HIP kernel's shape
+    r = Runner(ocn, torch_gpu, x, w)
+    try:
+        ocn.set_operand_precision(ocn.F16)
+        ocn.set_kernel_variant(ocn.KERNEL_ASM)
+        with pytest.raises(ocn.OpenCNNError):
+            r.dropin()
+        ocn.set_kernel_variant(ocn.KERNEL_AUTO)
+        assert not np.isnan(r.dropin()).any()
+    finally:
+        ocn.set_kernel_variant(ocn.KERNEL_AUTO)
+        ocn.set_operand_precision(ocn.F32)
+
+
 def test_reduced_precision_rejects_unsupported_shapes(ocn, torch_gpu):
     x, w = make_tensors(ocn, 32, 8, 6, 6, 64)  # C % 16 != 0
     r = Runner(ocn, torch_gpu, x, w)
