@@ -91,6 +91,76 @@ class KernelH16(Kernel):
         self.S["Kbf"] = S.get("Kbf")
         self.sgpr_count = S.next
 
+    def head(self):
+        """After the common set-up: the time-aligned chunk order.  A workgroup's g-th unit works on
+        chunk g mod Chunks of its tile, so that all workgroups (they start together) are at the
+        same chunk index at the same time and neighbouring tiles find their shared patch
+        columns and rows in L2.  The sum over the chunks of a tile does not care about the
+        order; a tile cut between two workgroups is shared as: the workgroup whose range starts
+        inside it takes chunks 0 .. N1-1 (its first units, in step with everybody), the one
+        whose range ends inside it takes the last Nlast chunks (the only units out of step).
+          N1     units of the first tile (Chunks when the range starts with a whole tile)
+          Sfull  N1 mod Chunks: the chunk index at which every later tile of the range starts
+          Tlast  last tile of the range, Nlast its units
+        They live in argument registers that are dead after this set-up."""
+        super().head()
+        t, e = self.t, self.e
+        self.S.update(N1=self.S["Kreal"], Sfull=self.S["UnitsQ"], Tlast=self.S["UnitsRem"], Nlast=self.S["Mch"])
+        e(f"s_add_u32 {t(2)}, {self.sr('Begin')}, {self.sr('Nunits')}")
+        e(f"s_sub_u32 {t(2)}, {t(2)}, 1")
+        self.div(t(3), t(2), self.sr("Mch"), self.sr("Sch"))  # before Mch is reused
+        e(f"s_sub_u32 {t(0)}, {self.sr('Chunks')}, {self.sr('Cm')}")
+        e(f"s_cmp_eq_u32 {self.sr('Cm')}, 0")
+        e(f"s_cselect_b32 {self.sr('N1')}, {self.sr('Chunks')}, {t(0)}")
+        e(f"s_cselect_b32 {self.sr('Sfull')}, 0, {t(0)}")
+        e(f"s_mov_b32 {self.sr('Tlast')}, {t(3)}")
+        e(f"s_mul_i32 {t(0)}, {t(3)}, {self.sr('Chunks')}")
+        e(f"s_sub_u32 {t(0)}, {t(2)}, {t(0)}")
+        e(f"s_add_u32 {self.sr('Nlast')}, {t(0)}, 1")
+        for n in ("Cm", "Cp", "Cq"):
+            e(f"s_mov_b32 {self.sr(n)}, 0")
+
+    def advance_cursor(self, T, C, ahead, hint, on_switch):
+        """Cursor (T, C) -> unit G+ahead when there is one: next chunk index modulo Chunks; the
+        tile ends where the index reaches Sfull (out of line: not inside the last tile), and the
+        last tile starts at Chunks - Nlast."""
+        rare, back = self.newlabel(hint + "_switch"), self.newlabel(hint + "_back")
+        t = self.t
+        self.e(f"s_add_u32 {t(0)}, {self.sr('G')}, {ahead}")
+        self.e(f"s_cmp_lt_u32 {t(0)}, {self.sr('Nunits')}")
+        self.e(f"s_addc_u32 {C}, {C}, 0")
+        self.e(f"s_cmp_eq_u32 {C}, {self.sr('Chunks')}")
+        self.e(f"s_cselect_b32 {C}, 0, {C}")
+        self.e(f"s_cmp_eq_u32 {C}, {self.sr('Sfull')}")
+        self.e(f"s_cbranch_scc1 {rare}")
+        self.label(back)
+        main, self.lines = self.lines, []
+        self.label(rare)
+        self.e(f"s_cmp_eq_u32 {T}, {self.sr('Tlast')}")
+        self.e(f"s_cbranch_scc1 {back}")
+        self.e(f"s_add_u32 {T}, {T}, 1")
+        self.e(f"s_sub_u32 {t(0)}, {self.sr('Chunks')}, {self.sr('Nlast')}")
+        self.e(f"s_cmp_eq_u32 {T}, {self.sr('Tlast')}")
+        self.e(f"s_cselect_b32 {C}, {t(0)}, {C}")
+        on_switch()
+        self.e(f"s_branch {back}")
+        self.outofline.extend(self.lines)
+        self.lines = main
+
+    def advance_p(self, ahead=3):
+        def switch():
+            self.decode(self.sr("Tp"))
+            self.patch_offsets()
+        self.advance_cursor(self.sr("Tp"), self.sr("Cp"), ahead, "p", switch)
+
+    def advance_q(self):
+        def switch():
+            t = self.t
+            self.filter_block(t(0), self.sr("Tq"))
+            self.e(f"s_lshl_b32 {t(0)}, {t(0)}, 2")
+            self.e(f"s_add_u32 {self.sr('KgQ')}, {t(0)}, {self.sr('Kw')}")
+        self.advance_cursor(self.sr("Tq"), self.sr("Cq"), 1, "q", switch)
+
     def range_owner(self):
         t = self.t
         self.e(f"s_cmp_eq_u32 {self.sr('Creal')}, 0")
@@ -307,6 +377,8 @@ class KernelH16(Kernel):
         self.end_of_chunk()
         self.e(f"s_add_u32 {self.sr('G')}, {self.sr('G')}, 1")
         self.e(f"s_add_u32 {self.sr('Cm')}, {self.sr('Cm')}, 1")
+        self.e(f"s_cmp_eq_u32 {self.sr('Cm')}, {self.sr('Chunks')}")
+        self.e(f"s_cselect_b32 {self.sr('Cm')}, 0, {self.sr('Cm')}")
 
     def resolve(self, ops, first):
         """Emit the chunk with its s_waitcnt counts.  vmcnt: memory instructions issued after the
@@ -384,14 +456,25 @@ class KernelH16(Kernel):
         check = [self.newlabel("check0"), self.newlabel("check1")]
         self.stamp()
         self.label(seg_loop)
-        e(f"s_sub_u32 {t(0)}, {self.sr('Nunits')}, {self.sr('G')}")
-        e(f"s_sub_u32 {t(1)}, {self.sr('Chunks')}, {self.sr('Cm')}")
-        e(f"s_min_u32 {t(0)}, {t(0)}, {t(1)}")
-        e(f"s_add_u32 {self.sr('SegEnd')}, {self.sr('Cm')}, {t(0)}")
-        e(f"s_cmp_lg_u32 {self.sr('Cm')}, 0")
+        # this segment: the units of tile Tm that belong to this workgroup; SegEnd in units of G.
+        # Kind: 1 publish (the range starts inside the tile), 2 merge (it ends inside), 0 whole tile.
+        e(f"s_cmp_eq_u32 {self.sr('G')}, 0")
+        e(f"s_cselect_b32 {t(0)}, {self.sr('N1')}, {self.sr('Chunks')}")
+        e(f"s_cmp_lt_u32 {t(0)}, {self.sr('Chunks')}")
         e(f"s_cselect_b32 {self.sr('Kind')}, 1, 0")
-        e(f"s_cmp_lt_u32 {self.sr('SegEnd')}, {self.sr('Chunks')}")
-        e(f"s_cbranch_scc0 {plain_seg}")
+        e(f"s_cmp_eq_u32 {self.sr('G')}, 0")   # a range's first tile is never its last partial one
+        e(f"s_cselect_b32 {t(1)}, -1, {self.sr('Tlast')}")
+        e(f"s_cmp_eq_u32 {self.sr('Tm')}, {t(1)}")
+        e(f"s_cselect_b32 {t(0)}, {self.sr('Nlast')}, {t(0)}")
+        e(f"s_sub_u32 {t(1)}, {self.sr('Nunits')}, {self.sr('G')}")
+        e(f"s_min_u32 {t(0)}, {t(0)}, {t(1)}")
+        e(f"s_add_u32 {self.sr('SegEnd')}, {self.sr('G')}, {t(0)}")
+        e(f"s_cmp_lt_u32 {t(0)}, {self.sr('Chunks')}")
+        e(f"s_cselect_b32 {t(1)}, 1, 0")
+        e(f"s_cmp_eq_u32 {self.sr('Kind')}, 1")
+        e(f"s_cselect_b32 {t(1)}, 0, {t(1)}")   # short and not the publishing one: the merging one
+        e(f"s_cmp_eq_u32 {t(1)}, 0")
+        e(f"s_cbranch_scc1 {plain_seg}")
         e(f"s_mov_b32 {self.sr('Kind')}, 2")
         self.merge_init()
         for kind, entry in (("merge", None), (True, plain_seg)):
@@ -407,11 +490,11 @@ class KernelH16(Kernel):
             e(f"s_branch {check[0]}")
         # steady state: even chunk, odd chunk, ...
         self.label(check[0])
-        e(f"s_cmp_lt_u32 {self.sr('Cm')}, {self.sr('SegEnd')}")
+        e(f"s_cmp_lt_u32 {self.sr('G')}, {self.sr('SegEnd')}")
         e(f"s_cbranch_scc0 {epi}")
         self.chunk(False, 0)
         self.label(check[1])
-        e(f"s_cmp_lt_u32 {self.sr('Cm')}, {self.sr('SegEnd')}")
+        e(f"s_cmp_lt_u32 {self.sr('G')}, {self.sr('SegEnd')}")
         e(f"s_cbranch_scc0 {epi}")
         self.chunk(False, 1)
         e(f"s_branch {check[0]}")
@@ -433,7 +516,9 @@ class KernelH16(Kernel):
         e(f"s_cmp_lt_u32 {self.sr('G')}, {self.sr('Nunits')}")
         e(f"s_cbranch_scc0 {done}")
         e(f"s_add_u32 {self.sr('Tm')}, {self.sr('Tm')}, 1")
-        e(f"s_mov_b32 {self.sr('Cm')}, 0")
+        e(f"s_sub_u32 {t(0)}, {self.sr('Chunks')}, {self.sr('Nlast')}")
+        e(f"s_cmp_eq_u32 {self.sr('Tm')}, {self.sr('Tlast')}")
+        e(f"s_cselect_b32 {self.sr('Cm')}, {t(0)}, {self.sr('Cm')}")  # else it is at Sfull already
         self.decode(self.sr("Tm"))
         self.m_tile_setup()
         e(f"s_branch {seg_loop}")
