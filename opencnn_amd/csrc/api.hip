@@ -249,9 +249,10 @@ int asm_grid(const opencnn::ConvArgs& a, int kw, int chunks, int* grid) {
 // order; fp16 / bf16: filter blocks, column-block major order).
 // lockstep_log2 >= 0 (fp16 / bf16 kernels only): one line of units per filter block, 2^lockstep_log2
 // filter blocks; tile_split is then their number and c_real (the mode flag of those kernels) 0.
+// epilogue_weight >= 0 (fp16 / bf16 kernels only): cost of an output transform in half units.
 int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmKernels* ak, hipFunction_t fn, int chunks,
-                      long long usw_bytes, int tile_split, int c_real, int lockstep_log2, int grid,
-                      size_t lds_bytes, hipStream_t st) {
+                      long long usw_bytes, int tile_split, int c_real, int lockstep_log2,
+                      int epilogue_weight, int grid, size_t lds_bytes, hipStream_t st) {
   AsmKernArgs ka{};
   ka.x = a.x;
   ka.usw = a.usw;
@@ -275,12 +276,22 @@ int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmKernels* ak, hipFunct
     total >>= lockstep_log2;
     ranges >>= lockstep_log2;
   }
+  uint32_t chunk_divisor = (uint32_t)chunks;
+  if (epilogue_weight >= 0) {
+    // fp16 / bf16 kernels: ranges are cut on a weighted line in half units, a tile = its chunks
+    // plus the cost of its output transform (the kernel maps a weighted position back to a unit)
+    const long long vt = 2LL * chunks + epilogue_weight;
+    total = total / chunks * vt;
+    if (total > kMaxElems) return fail("weighted unit line below 2^31");
+    ka.k_real = (int32_t)vt;
+    chunk_divisor = (uint32_t)vt;
+  }
   ka.units_q = (int32_t)(total / ranges);
   ka.units_rem = (int32_t)(total % ranges);
   ka.usw_bytes = (int32_t)usw_bytes;
   ka.grid_per_xcd = grid % 8 == 0 ? grid / 8 : 0;  // 0: no XCD-aware block order
   ka.timeline = (size_t)grid * 64 * sizeof(long long) <= g_timeline_bytes.load() ? g_timeline.load() : nullptr;
-  magic_divisor((uint32_t)chunks, &ka.m_chunks, &ka.s_chunks);
+  magic_divisor(chunk_divisor, &ka.m_chunks, &ka.s_chunks);
   magic_divisor((uint32_t)tile_split, &ka.m_colblocks, &ka.s_colblocks);
   if (lockstep_log2 >= 0) ka.s_colblocks = (uint32_t)lockstep_log2;
   magic_divisor((uint32_t)a.ngroups, &ka.m_ngroups, &ka.s_ngroups);
@@ -299,11 +310,14 @@ int launch_asm(const opencnn::ConvArgs& a, int kw, int grid, bool ragged, size_t
   const hipFunction_t fn =
       ragged ? (kw == 4 ? ak->kw4_ragged : ak->kw2_ragged) : (kw == 4 ? ak->kw4 : ak->kw2);
   return launch_asm_kernel(a, ak, fn, (a.C + 7) / 8, padded_c(a.C) * 16 * padded_k(a.K) * 4, a.colblocks,
-                           a.C, -1, grid, lds_bytes, st);
+                           a.C, -1, -1, grid, lds_bytes, st);
 }
 
 // The hand-scheduled fp16 / bf16 kernels (gen_wino_h16_asm.py) take whole 128-filter blocks and
 // 16-channel chunks of shapes inside the reference's tiling; *launched stays false otherwise.
+// An output transform of the fp16 / bf16 kernels takes about as long as 1.5 of their units.
+constexpr int kEpilogueHalfUnits = 3;
+
 int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* launched) {
   *launched = false;
   if (a.N % 32 != 0 || a.C % 16 != 0 || a.K % 128 != 0) return 0;
@@ -328,8 +342,8 @@ int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* lau
   int log2k = 0;
   while ((1 << log2k) < kblocks) ++log2k;
   const bool lockstep = usw_bytes <= (2 << 20) && (1 << log2k) == kblocks && grid % kblocks == 0;
-  const int e = lockstep ? launch_asm_kernel(a, ak, fn, chunks, usw_bytes, kblocks, 0, log2k, grid, lds_bytes, st)
-                         : launch_asm_kernel(a, ak, fn, chunks, usw_bytes, a.colblocks, 1, -1, grid, lds_bytes, st);
+  const int e = lockstep ? launch_asm_kernel(a, ak, fn, chunks, usw_bytes, kblocks, 0, log2k, kEpilogueHalfUnits, grid, lds_bytes, st)
+                         : launch_asm_kernel(a, ak, fn, chunks, usw_bytes, a.colblocks, 1, -1, kEpilogueHalfUnits, grid, lds_bytes, st);
   *launched = e == 0;
   return e;
 }

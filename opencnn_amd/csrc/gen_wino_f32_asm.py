@@ -677,6 +677,20 @@ class Kernel:
         """The register that numbers this workgroup's range of units."""
         return self.sr("L")
 
+    def unit_range(self, owner):
+        """Begin, Nunits (units [Begin, Begin + Nunits): the first UnitsRem ranges take one more)
+        and the first unit's tile Tm and chunk Cm."""
+        t, e = self.t, self.e
+        e(f"s_mul_i32 {self.sr('Begin')}, {owner}, {self.sr('UnitsQ')}")
+        e(f"s_min_u32 {t(0)}, {owner}, {self.sr('UnitsRem')}")
+        e(f"s_add_u32 {self.sr('Begin')}, {self.sr('Begin')}, {t(0)}")
+        e(f"s_cmp_lt_u32 {owner}, {self.sr('UnitsRem')}")
+        e(f"s_cselect_b32 {t(0)}, 1, 0")
+        e(f"s_add_u32 {self.sr('Nunits')}, {self.sr('UnitsQ')}, {t(0)}")
+        self.div(self.sr("Tm"), self.sr("Begin"), self.sr("Mch"), self.sr("Sch"))
+        e(f"s_mul_i32 {t(0)}, {self.sr('Tm')}, {self.sr('Chunks')}")
+        e(f"s_sub_u32 {self.sr('Cm')}, {self.sr('Begin')}, {t(0)}")
+
     def head(self):
         """Kernel arguments, wave / workgroup identity, the unit range, cursors, descriptors."""
         S, t = self.S, self.t
@@ -708,17 +722,7 @@ class Kernel:
         e(f"s_add_u32 {t(0)}, {t(0)}, {t(1)}")
         e(f"s_cmp_eq_u32 {self.sr('GridPerXcd')}, 0")
         e(f"s_cselect_b32 {self.sr('L')}, s2, {t(0)}")
-        # units [Begin, Begin + Nunits): the first UnitsRem blocks take one more
-        owner = self.range_owner()
-        e(f"s_mul_i32 {self.sr('Begin')}, {owner}, {self.sr('UnitsQ')}")
-        e(f"s_min_u32 {t(0)}, {owner}, {self.sr('UnitsRem')}")
-        e(f"s_add_u32 {self.sr('Begin')}, {self.sr('Begin')}, {t(0)}")
-        e(f"s_cmp_lt_u32 {owner}, {self.sr('UnitsRem')}")
-        e(f"s_cselect_b32 {t(0)}, 1, 0")
-        e(f"s_add_u32 {self.sr('Nunits')}, {self.sr('UnitsQ')}, {t(0)}")
-        self.div(self.sr("Tm"), self.sr("Begin"), self.sr("Mch"), self.sr("Sch"))
-        e(f"s_mul_i32 {t(0)}, {self.sr('Tm')}, {self.sr('Chunks')}")
-        e(f"s_sub_u32 {self.sr('Cm')}, {self.sr('Begin')}, {t(0)}")
+        self.unit_range(self.range_owner())
         for n in ("Tp", "Tq"):
             e(f"s_mov_b32 {self.sr(n)}, {self.sr('Tm')}")
         for n in ("Cp", "Cq"):

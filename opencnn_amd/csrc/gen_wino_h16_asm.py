@@ -101,22 +101,15 @@ class KernelH16(Kernel):
         whose range ends inside it takes the last Nlast chunks (the only units out of step).
           N1     units of the first tile (Chunks when the range starts with a whole tile)
           Sfull  N1 mod Chunks: the chunk index at which every later tile of the range starts
-          Tlast  last tile of the range, Nlast its units
+          Tlast  last tile of the range, Nlast its units (both left by unit_range)
         They live in argument registers that are dead after this set-up."""
         super().head()
         t, e = self.t, self.e
         self.S.update(N1=self.S["Kreal"], Sfull=self.S["UnitsQ"], Tlast=self.S["UnitsRem"], Nlast=self.S["Mch"])
-        e(f"s_add_u32 {t(2)}, {self.sr('Begin')}, {self.sr('Nunits')}")
-        e(f"s_sub_u32 {t(2)}, {t(2)}, 1")
-        self.div(t(3), t(2), self.sr("Mch"), self.sr("Sch"))  # before Mch is reused
         e(f"s_sub_u32 {t(0)}, {self.sr('Chunks')}, {self.sr('Cm')}")
         e(f"s_cmp_eq_u32 {self.sr('Cm')}, 0")
         e(f"s_cselect_b32 {self.sr('N1')}, {self.sr('Chunks')}, {t(0)}")
         e(f"s_cselect_b32 {self.sr('Sfull')}, 0, {t(0)}")
-        e(f"s_mov_b32 {self.sr('Tlast')}, {t(3)}")
-        e(f"s_mul_i32 {t(0)}, {t(3)}, {self.sr('Chunks')}")
-        e(f"s_sub_u32 {t(0)}, {t(2)}, {t(0)}")
-        e(f"s_add_u32 {self.sr('Nlast')}, {t(0)}, 1")
         for n in ("Cm", "Cp", "Cq"):
             e(f"s_mov_b32 {self.sr(n)}, 0")
 
@@ -160,6 +153,48 @@ class KernelH16(Kernel):
             self.e(f"s_lshl_b32 {t(0)}, {t(0)}, 2")
             self.e(f"s_add_u32 {self.sr('KgQ')}, {t(0)}, {self.sr('Kw')}")
         self.advance_cursor(self.sr("Tq"), self.sr("Cq"), 1, "q", switch)
+
+    def unit_range(self, owner):
+        """The ranges are cut on a weighted line: a tile counts 2 * Chunks for its units plus the
+        cost of its output transform in half units (a unit here is four times shorter than an
+        fp32 one, so a range with one more tile end would otherwise finish 2 us late).  VT = the
+        weighted length of a tile arrives in the argument slot of the ragged kernels' real filter
+        count, its magic number in (Mch, Sch); UnitsQ / UnitsRem count weighted half units.
+        Weighted position v -> tile v / VT, chunk min((v % VT + 1) / 2, Chunks)."""
+        t, e = self.t, self.e
+        vt = self.sr("Kreal")
+        for which, dst in ((0, self.sr("Begin")), (1, t(5))):
+            if which:
+                e(f"s_add_u32 {t(0)}, {owner}, 1")
+            else:
+                e(f"s_mov_b32 {t(0)}, {owner}")
+            e(f"s_mul_i32 {t(1)}, {t(0)}, {self.sr('UnitsQ')}")
+            e(f"s_min_u32 {t(2)}, {t(0)}, {self.sr('UnitsRem')}")
+            e(f"s_add_u32 {t(1)}, {t(1)}, {t(2)}")          # weighted start of range `owner + which`
+            self.div(t(2), t(1), self.sr("Mch"), self.sr("Sch"))  # tile
+            e(f"s_mul_i32 {t(3)}, {t(2)}, {vt}")
+            e(f"s_sub_u32 {t(3)}, {t(1)}, {t(3)}")
+            e(f"s_add_u32 {t(3)}, {t(3)}, 1")
+            e(f"s_lshr_b32 {t(3)}, {t(3)}, 1")
+            e(f"s_min_u32 {t(3)}, {t(3)}, {self.sr('Chunks')}")  # chunk
+            if not which:
+                e(f"s_mov_b32 {self.sr('Tm')}, {t(2)}")
+                e(f"s_mov_b32 {self.sr('Cm')}, {t(3)}")
+            else:
+                e(f"s_mov_b32 {t(4)}, {t(2)}")
+            e(f"s_mul_i32 {t(2)}, {t(2)}, {self.sr('Chunks')}")
+            e(f"s_add_u32 {dst}, {t(2)}, {t(3)}")
+        e(f"s_sub_u32 {self.sr('Nunits')}, {t(5)}, {self.sr('Begin')}")
+        # the range ends in front of (tile T4, chunk T3): its last tile and the units it has there.
+        # They replace UnitsRem and Mch, which are dead from here on (see head).
+        e(f"s_sub_u32 {t(0)}, {t(4)}, 1")
+        e(f"s_cmp_eq_u32 {t(3)}, 0")
+        e(f"s_cselect_b32 {self.sr('UnitsRem')}, {t(0)}, {t(4)}")
+        e(f"s_cselect_b32 {self.sr('Mch')}, {self.sr('Chunks')}, {t(3)}")
+        # a weighted start that falls on a tile's last chunk boundary is the next tile's first unit
+        e(f"s_cmp_eq_u32 {self.sr('Cm')}, {self.sr('Chunks')}")
+        e(f"s_cselect_b32 {self.sr('Cm')}, 0, {self.sr('Cm')}")
+        e(f"s_addc_u32 {self.sr('Tm')}, {self.sr('Tm')}, 0")
 
     def range_owner(self):
         t = self.t
