@@ -45,6 +45,7 @@ MEASURED_TRAFFIC_BYTES = {
     "resnet_n128_c128_h28_k128": 261.3e6,
     "deep_n128_c256_h14_k256": 250.1e6,
     "deep_n128_c512_h7_k512": 112.7e6,
+    "reduced_n128_c256_h14_k256_f16": 165.5e6,
 }
 
 
@@ -123,22 +124,24 @@ def miopen_column(torch, lay, warmup=10, iters=200, settle_ms=150.0):
     return ev[0].elapsed_time(ev[1]) / iters
 
 
-def timeline_summary(ocn, torch, lay, launches=20):
+def timeline_summary(ocn, torch, lay, launches=20, operands="f32"):
     """Where a launch of the assembly kernels spends its time: per-workgroup stamps (kernel start,
     end of the prologue, before / after every output transform) of the last of `launches`
     back-to-back launches with pre-transformed filters, summarised in microseconds."""
     import numpy as np
 
     o = lay
-    ocn.filter_transform(o.w, o.ws, o.K, o.C, ocn.FILTER_CRSK, ocn.WW_MFMA)
     buf = torch.zeros(1024 * 64, dtype=torch.int64, device=o.x.device)
     try:
+        ocn.set_operand_precision({"f32": ocn.F32, "f16": ocn.F16, "bf16": ocn.BF16}[operands])
+        ocn.filter_transform(o.w, o.ws, o.K, o.C, ocn.FILTER_CRSK, ocn.WW_MFMA)
         ocn.set_timeline_buffer(buf)
         for _ in range(launches):
             ocn.conv_forward_pretransformed(o.x, o.ws, o.y, o.N, o.C, o.H, o.H, o.K)
         torch.cuda.synchronize()
     finally:
         ocn.set_timeline_buffer(None)
+        ocn.set_operand_precision(ocn.F32)
     nwg = int((buf.cpu().numpy().reshape(-1, 64)[:, 0] > 0).sum())
     if nwg == 0:
         return {"workload": o.name, "recorded_workgroups": 0}
@@ -150,7 +153,7 @@ def timeline_summary(ocn, torch, lay, launches=20):
         segs += d[1::2].tolist()
         epis += d[2::2].tolist()
     segs, epis = np.array(segs), np.array(epis)
-    chunks = o.C // 8
+    chunks = o.C // (8 if operands == "f32" else 16)
     return {
         "workload": o.name, "recorded_workgroups": nwg,
         "kernel_span_us": float(ends.max()),
@@ -191,7 +194,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(FP32_LAYERS))
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(LAYERS))
+    ap.add_argument("--operands", default="f32", choices=["f32", "f16", "bf16"],
+                    help="GEMM operand precision of the timed workload (fp32 transforms and "
+                         "accumulation in every case); the default is the reference's fp32")
     ap.add_argument("--settle-ms", type=float, default=300.0,
                     help="untimed back-to-back run before every measurement (0: measure from idle)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -217,6 +223,10 @@ def main():
 
     layer = Layer(ocn, torch, args.workload)
     fd, fm, bmin = work(layer.N, layer.C, layer.H, layer.K)
+    reduced = args.operands != "f32"
+    if reduced:
+        ocn.set_operand_precision(ocn.F16 if args.operands == "f16" else ocn.BF16)
+    peak = PEAK_F16_MFMA_TFLOPS if reduced else PEAK_FP32_MFMA_TFLOPS
 
     settle(torch, layer, args.settle_ms)
     for _ in range(args.warmup):
@@ -232,10 +242,11 @@ def main():
     # dominant kernel, HIP events on the launch stream, same number of launches
     _, ms_main, ms_fx = layer.kernel_times(args.warmup, args.steps)
     achieved = fm / (ms_main * 1e-3) / 1e12
-    traffic = MEASURED_TRAFFIC_BYTES.get(layer.name)
+    traffic = MEASURED_TRAFFIC_BYTES.get(layer.name + ("_" + args.operands if reduced else ""))
+    ocn.set_operand_precision(ocn.F32)
 
     out = {
-        "metric": "effective TFLOP/s (direct-conv FLOPs 2*N*K*C*H*W*9) of one 3x3 fp32 layer, "
+        "metric": "effective TFLOP/s (direct-conv FLOPs 2*N*K*C*H*W*9) of one 3x3 layer, "
                   "filter transform + fused Winograd kernel per call",
         "value": fd / (ms_step * 1e-3) / 1e12,
         "unit": "TFLOP/s",
@@ -247,18 +258,19 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": args.operands,
         "data": "synthetic",
         "config": {"workload": layer.name, "N": layer.N, "C": layer.C, "H": layer.H,
                    "W": layer.H, "K": layer.K, "pad": 1, "stride": 1,
                    "layout": "CHWN in, CRSK filters, KHWN out"},
         "roofline": {
-            "kernel": "wino_f32_asm_kw2 / wino_f32_asm_kw4 (fused Winograd kernel, hand-scheduled assembly)",
+            "kernel": ("wino_f16_asm_kw4 / wino_bf16_asm_kw4" if reduced else "wino_f32_asm_kw2 / wino_f32_asm_kw4") +
+                      " (fused Winograd kernel, hand-scheduled assembly)",
             "bound": "mfma",
             "achieved": achieved,
-            "peak": PEAK_FP32_MFMA_TFLOPS,
+            "peak": peak,
             "unit": "TFLOP/s",
-            "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
+            "frac": achieved / peak,
             "traffic": traffic,
             "flops_per_launch": fm,
             "ms_per_launch": ms_main,
@@ -275,11 +287,11 @@ def main():
         out["cpu_baseline"] = base
         rel, max_abs, max_ref = oracle.compare(layer.y.cpu().numpy(), y_ref)
         out["check"] = {"rel_l2_vs_fp64_direct": rel, "max_abs": max_abs, "max_ref": max_ref}
-        if not rel <= 1e-3:
+        if not rel <= (1.5e-2 if reduced else 1e-3):
             sys.exit(f"bench.py: GPU result differs from the fp64 direct convolution (rel-L2 {rel})")
 
     if args.timeline:
-        out["timeline"] = [timeline_summary(ocn, torch, layer)]
+        out["timeline"] = [timeline_summary(ocn, torch, layer, operands=args.operands)]
 
     if not args.no_layers:
         rows = []
