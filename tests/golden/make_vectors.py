@@ -9,9 +9,11 @@ in exact int64 arithmetic with numpy only (KHWN).  Every product and sum is exac
 representable in fp32, so a correct fp32 implementation, Winograd or not, must reproduce the
 stored outputs bit for bit.
 
-Usage: python tests/golden/make_vectors.py   (rewrites the .npz files next to it)
+Usage: python tests/golden/make_vectors.py [name ...]   (rewrites the named .npz files next to it,
+all of them without arguments)
 """
 import os
+import sys
 
 import numpy as np
 
@@ -22,6 +24,9 @@ CASES = {
     "int_n32_c8_h5_w6_k64": (32, 8, 5, 6, 64, 1),      # odd / even sides, one chunk
     "int_n32_c24_h9_w9_k128": (32, 24, 9, 9, 128, 2),  # three chunks, four filter groups
     "int_n33_c5_h4_w7_k40": (33, 5, 4, 7, 40, 3),      # outside the reference's tiling
+    # two 16-channel chunks, a 128-filter block: also a shape of the fp16 / bf16 kernels, whose
+    # roundings are exact on these values too (|U| <= 18, |V| <= 16)
+    "int_n32_c32_h7_w7_k128": (32, 32, 7, 7, 128, 4),
 }
 
 
@@ -40,6 +45,8 @@ def direct_conv_int(x, w):
 
 def main():
     for name, (N, C, H, W, K, seed) in CASES.items():
+        if sys.argv[1:] and name not in sys.argv[1:]:
+            continue
         rng = np.random.default_rng(seed)
         # multiples of 1/4 would survive G g G^T exactly as well; integers keep the file small
         x = rng.integers(-4, 5, size=(C, H, W, N)).astype(np.int8)

@@ -197,3 +197,7 @@ def test_oracle_reproduces_known_answer_vectors(oracle, name):
     assert np.array_equal(oracle.direct_conv_f64(x, w), y.astype(np.float64))
     if x.shape[1] == x.shape[2]:  # the restatement follows the reference: square images only
         assert np.array_equal(oracle.winograd_f32(x, w), y.astype(np.float32))
+        # the fp16 / bf16 roundings of the quantised restatement are exact on these values
+        # (|U| <= 18, |V| <= 16 are integers), so it must hit the same vectors
+        assert np.array_equal(oracle.winograd_f32(x, w, 1), y.astype(np.float32))
+        assert np.array_equal(oracle.winograd_f32(x, w, 2), y.astype(np.float32))

@@ -197,6 +197,26 @@ def test_known_answer_vectors_bit_exact(ocn, torch_gpu, name, family):
     assert np.array_equal(y, want)
 
 
+@pytest.mark.parametrize("prec", ["f16", "bf16"])
+@pytest.mark.parametrize("family", ["auto", "hip"])
+def test_known_answer_vector_bit_exact_with_reduced_operands(ocn, torch_gpu, family, prec):
+    # small integers survive the fp16 / bf16 roundings of U and V unchanged (|U| <= 18, |V| <= 16),
+    # so the reduced-precision kernels must reproduce the committed vector bit for bit as well
+    name = "int_n32_c32_h7_w7_k128"
+    print(f"golden {name} {family} {prec}", flush=True)
+    v = np.load(os.path.join(GOLDEN, name + ".npz"))
+    x, w, want = v["x"].astype(np.float32), v["w"].astype(np.float32), v["y"].astype(np.float32)
+    r = Runner(ocn, torch_gpu, x, w)
+    try:
+        ocn.set_operand_precision(ocn.F16 if prec == "f16" else ocn.BF16)
+        ocn.set_kernel_variant(ocn.KERNEL_AUTO if family == "auto" else ocn.KERNEL_HIP)
+        y = r.split()
+    finally:
+        ocn.set_kernel_variant(ocn.KERNEL_AUTO)
+        ocn.set_operand_precision(ocn.F32)
+    assert np.array_equal(y, want)
+
+
 def test_impulse_reproduces_filter_taps(ocn, torch_gpu):
     # one non-zero input pixel: y[:, h0-(r-1), w0-(s-1), n0] = g[c0][r][s][:]; pins all strides
     print("impulse", flush=True)
