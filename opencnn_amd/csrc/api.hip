@@ -244,15 +244,27 @@ int asm_grid(const opencnn::ConvArgs& a, int kw, int chunks, int* grid) {
   return 0;
 }
 
-// chunks: units per workgroup tile; usw_bytes: size of the transformed filter; tile_split: the
-// divisor that takes a workgroup tile index apart (fp32: column blocks, filter-block major
-// order; fp16 / bf16: filter blocks, column-block major order).
-// lockstep_log2 >= 0 (fp16 / bf16 kernels only): one line of units per filter block, 2^lockstep_log2
-// filter blocks; tile_split is then their number and c_real (the mode flag of those kernels) 0.
-// epilogue_weight >= 0 (fp16 / bf16 kernels only): cost of an output transform in half units.
-int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmKernels* ak, hipFunction_t fn, int chunks,
-                      long long usw_bytes, int tile_split, int c_real, int lockstep_log2,
-                      int epilogue_weight, int grid, size_t lds_bytes, hipStream_t st) {
+// One launch of a hand-scheduled kernel.
+struct AsmLaunch {
+  hipFunction_t fn = nullptr;
+  int grid = 0;
+  size_t lds_bytes = 0;
+  int chunks = 0;           // units per workgroup tile
+  long long usw_bytes = 0;  // size of the transformed filter
+  // The divisor that takes a workgroup tile index apart: the column blocks (filter-block major
+  // line of units), or, with lockstep_log2 >= 0, the filter blocks.
+  int tile_split = 1;
+  // fp32 kernels: the real channel count (ragged shapes).  fp16 / bf16 kernels: 0 = one line of
+  // units per filter block (2^lockstep_log2 of them, walked in lockstep), 1 = one line.
+  int c_real_or_mode = 0;
+  int lockstep_log2 = -1;
+  // fp16 / bf16 kernels (>= 0): cost of an output transform in half units; ranges are then cut on
+  // a weighted line, a tile = 2 * chunks + this, and the kernel maps positions back to units.
+  int epilogue_half_units = -1;
+};
+
+int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmKernels* ak, const AsmLaunch& l, hipStream_t st) {
+  const int chunks = l.chunks, grid = l.grid;
   AsmKernArgs ka{};
   ka.x = a.x;
   ka.usw = a.usw;
@@ -265,22 +277,20 @@ int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmKernels* ak, hipFunct
   ka.tiles_w = a.tiles_w;
   ka.ngroups = a.ngroups;
   ka.colgroups = a.colgroups;
-  ka.colblocks = tile_split;
+  ka.colblocks = l.tile_split;
   ka.Q = chunks * 2;
   ka.HWN4 = a.N * a.H * a.W * 4;
-  ka.c_real = c_real;
+  ka.c_real = l.c_real_or_mode;
   ka.k_real = a.K;
   long long total = (long long)a.nblocks * chunks;
   int ranges = grid;
-  if (lockstep_log2 >= 0) {
-    total >>= lockstep_log2;
-    ranges >>= lockstep_log2;
+  if (l.lockstep_log2 >= 0) {
+    total >>= l.lockstep_log2;
+    ranges >>= l.lockstep_log2;
   }
   uint32_t chunk_divisor = (uint32_t)chunks;
-  if (epilogue_weight >= 0) {
-    // fp16 / bf16 kernels: ranges are cut on a weighted line in half units, a tile = its chunks
-    // plus the cost of its output transform (the kernel maps a weighted position back to a unit)
-    const long long vt = 2LL * chunks + epilogue_weight;
+  if (l.epilogue_half_units >= 0) {
+    const long long vt = 2LL * chunks + l.epilogue_half_units;  // weighted length of a tile
     total = total / chunks * vt;
     if (total > kMaxElems) return fail("weighted unit line below 2^31");
     ka.k_real = (int32_t)vt;
@@ -288,18 +298,18 @@ int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmKernels* ak, hipFunct
   }
   ka.units_q = (int32_t)(total / ranges);
   ka.units_rem = (int32_t)(total % ranges);
-  ka.usw_bytes = (int32_t)usw_bytes;
+  ka.usw_bytes = (int32_t)l.usw_bytes;
   ka.grid_per_xcd = grid % 8 == 0 ? grid / 8 : 0;  // 0: no XCD-aware block order
   ka.timeline = (size_t)grid * 64 * sizeof(long long) <= g_timeline_bytes.load() ? g_timeline.load() : nullptr;
   magic_divisor(chunk_divisor, &ka.m_chunks, &ka.s_chunks);
-  magic_divisor((uint32_t)tile_split, &ka.m_colblocks, &ka.s_colblocks);
-  if (lockstep_log2 >= 0) ka.s_colblocks = (uint32_t)lockstep_log2;
+  magic_divisor((uint32_t)l.tile_split, &ka.m_colblocks, &ka.s_colblocks);
+  if (l.lockstep_log2 >= 0) ka.s_colblocks = (uint32_t)l.lockstep_log2;
   magic_divisor((uint32_t)a.ngroups, &ka.m_ngroups, &ka.s_ngroups);
   magic_divisor((uint32_t)a.tiles_w, &ka.m_tiles_w, &ka.s_tiles_w);
   size_t ka_size = sizeof(ka);
   void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &ka, HIP_LAUNCH_PARAM_BUFFER_SIZE, &ka_size,
                    HIP_LAUNCH_PARAM_END};
-  return (int)hipModuleLaunchKernel(fn, (unsigned)grid, 1, 1, 256, 1, 1, (unsigned)lds_bytes, st,
+  return (int)hipModuleLaunchKernel(l.fn, (unsigned)grid, 1, 1, 256, 1, 1, (unsigned)l.lds_bytes, st,
                                     nullptr, extra);
 }
 
@@ -307,10 +317,15 @@ int launch_asm(const opencnn::ConvArgs& a, int kw, int grid, bool ragged, size_t
                hipStream_t st) {
   const AsmKernels* ak = nullptr;
   if (int e = asm_kernels(&ak)) return e;
-  const hipFunction_t fn =
-      ragged ? (kw == 4 ? ak->kw4_ragged : ak->kw2_ragged) : (kw == 4 ? ak->kw4 : ak->kw2);
-  return launch_asm_kernel(a, ak, fn, (a.C + 7) / 8, padded_c(a.C) * 16 * padded_k(a.K) * 4, a.colblocks,
-                           a.C, -1, -1, grid, lds_bytes, st);
+  AsmLaunch l;
+  l.fn = ragged ? (kw == 4 ? ak->kw4_ragged : ak->kw2_ragged) : (kw == 4 ? ak->kw4 : ak->kw2);
+  l.grid = grid;
+  l.lds_bytes = lds_bytes;
+  l.chunks = (a.C + 7) / 8;
+  l.usw_bytes = padded_c(a.C) * 16 * padded_k(a.K) * 4;
+  l.tile_split = a.colblocks;
+  l.c_real_or_mode = a.C;
+  return launch_asm_kernel(a, ak, l, st);
 }
 
 // The hand-scheduled fp16 / bf16 kernels (gen_wino_h16_asm.py) take whole 128-filter blocks and
@@ -324,7 +339,9 @@ int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* lau
   if ((long long)a.N * a.H * a.W * 4 * 4 > kMaxElems) return 0;  // four-channel slab in bytes
   const int kblocks = a.kgroups / 4, chunks = a.C / 16;
   const long long nblocks = (long long)a.colgroups * kblocks;
-  if (nblocks > kMaxElems / 8) return 0;
+  const long long usw_bytes = (long long)a.C * 16 * a.K * 2;
+  if (nblocks > kMaxElems / 8 || usw_bytes > kMaxElems) return 0;
+  if (nblocks * (2LL * chunks + kEpilogueHalfUnits) > kMaxElems) return 0;  // the weighted line of units
   a.nblocks = (int)nblocks;
   a.colblocks = a.colgroups;
   int grid = 0;
@@ -332,18 +349,28 @@ int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* lau
   if (grid == 0) return 0;
   const AsmKernels* ak = nullptr;
   if (int e = asm_kernels(&ak)) return e;
-  const hipFunction_t fn = precision == OPENCNN_BF16 ? ak->bf16_kw4 : ak->f16_kw4;
-  const size_t lds_bytes = 2 * 16 * 2 * 4 * 32 * sizeof(unsigned);  // two buffers of V
+  AsmLaunch l;
+  l.fn = precision == OPENCNN_BF16 ? ak->bf16_kw4 : ak->f16_kw4;
+  l.grid = grid;
+  l.lds_bytes = 2 * 16 * 2 * 4 * 32 * sizeof(unsigned);  // two buffers of V
+  l.chunks = chunks;
+  l.usw_bytes = usw_bytes;
+  l.epilogue_half_units = kEpilogueHalfUnits;
   // How the units are dealt.  While the whole 2-byte transformed filter leaves room in an XCD's
   // 4 MB L2 and the filter blocks are a power of two that divides the grid: one line of units per
   // filter block, walked in lockstep by neighbouring workgroups (the patches the filter blocks
   // share are read from HBM once).  Else one filter-block-major line as in the fp32 kernels.
-  const long long usw_bytes = (long long)a.C * 16 * a.K * 2;
   int log2k = 0;
   while ((1 << log2k) < kblocks) ++log2k;
-  const bool lockstep = usw_bytes <= (2 << 20) && (1 << log2k) == kblocks && grid % kblocks == 0;
-  const int e = lockstep ? launch_asm_kernel(a, ak, fn, chunks, usw_bytes, kblocks, 0, log2k, kEpilogueHalfUnits, grid, lds_bytes, st)
-                         : launch_asm_kernel(a, ak, fn, chunks, usw_bytes, a.colblocks, 1, -1, kEpilogueHalfUnits, grid, lds_bytes, st);
+  if (usw_bytes <= (2 << 20) && (1 << log2k) == kblocks && grid % kblocks == 0) {
+    l.tile_split = kblocks;
+    l.c_real_or_mode = 0;
+    l.lockstep_log2 = log2k;
+  } else {
+    l.tile_split = a.colblocks;
+    l.c_real_or_mode = 1;
+  }
+  const int e = launch_asm_kernel(a, ak, l, st);
   *launched = e == 0;
   return e;
 }
