@@ -99,6 +99,42 @@ def settle(torch, lay, ms):
         torch.cuda.synchronize()
 
 
+def shim_rows(ocn, torch, lay, iters=200):
+    """The layout shims (NCHW -> CHWN, KHWN -> NKHW, KCRS -> CRSK; they replace the reference's
+    data_cpy, src/openCNN_winograd.cu:147-153) and the filter transform on this layer: HBM-bound
+    kernels, algorithmic bytes = one read + one write of every element (filter transform: 36 B
+    read + 64 B written per (c, k)).  Timed with events on the null stream, which is the stream the
+    library launches on unless opencnn_set_stream says otherwise."""
+    o = lay
+    dev = o.x.device
+    nchw = torch.rand((o.N, o.C, o.H, o.H), device=dev)
+    nkhw = torch.empty((o.N, o.K, o.H, o.H), device=dev)
+    kcrs = torch.rand((o.K, o.C, 3, 3), device=dev)
+    crsk = torch.empty((o.C, 3, 3, o.K), device=dev)
+    chwn = torch.empty_like(o.x)
+    cases = [
+        ("nchw_to_chwn", lambda: ocn.nchw_to_chwn(nchw, chwn, o.N, o.C, o.H, o.H), 8.0 * nchw.numel()),
+        ("khwn_to_nkhw", lambda: ocn.khwn_to_nkhw(o.y, nkhw, o.N, o.K, o.H, o.H), 8.0 * nkhw.numel()),
+        ("kcrs_to_crsk", lambda: ocn.kcrs_to_crsk(kcrs, crsk, o.K, o.C), 8.0 * kcrs.numel()),
+        ("filter_transform", lambda: ocn.filter_transform(o.w, o.ws, o.K, o.C, ocn.FILTER_CRSK, ocn.WW_MFMA),
+         100.0 * o.K * o.C),
+    ]
+    rows = []
+    for name, fn, nbytes in cases:
+        for _ in range(iters):  # also the settle phase of this kernel
+            fn()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        ev[0].record()
+        for _ in range(iters):
+            fn()
+        ev[1].record()
+        torch.cuda.synchronize()
+        ms = ev[0].elapsed_time(ev[1]) / iters
+        rows.append({"workload": o.name, "kernel": name, "us": ms * 1e3, "bytes": nbytes,
+                     "gbs": nbytes / (ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS})
+    return rows
+
+
 def miopen_column(torch, lay, warmup=10, iters=200, settle_ms=150.0):
     """Informational only, never an oracle: ms per call of torch.nn.functional.conv2d (MIOpen's
     own choice of fp32 algorithm) on the same layer in NCHW / KCRS, the analogue of the
@@ -205,6 +241,9 @@ def main():
     ap.add_argument("--timeline", action="store_true",
                     help="add the assembly kernels' per-workgroup timeline of the workload (and of every "
                          "fp32 layer of the table) to the output")
+    ap.add_argument("--shims", action="store_true",
+                    help="add the layout shims and the filter transform (HBM-bound kernels) of every "
+                         "fp32 layer to the output")
     ap.add_argument("--miopen", action="store_true",
                     help="add an informational MIOpen (torch conv2d, fp32) column to the per-layer table")
     args = ap.parse_args()
@@ -320,6 +359,8 @@ def main():
                     "mfma_frac_of_peak": m / (mn * 1e-3) / 1e12 / peak,
                     "hbm_gbs_at_min_bytes": b / (tot * 1e-3) / 1e9,
                 })
+            if args.shims and not name.startswith("reduced"):
+                out.setdefault("shims", []).extend(shim_rows(ocn, torch, lay))
             if args.timeline and name != layer.name and not name.startswith("reduced"):
                 out["timeline"].append(timeline_summary(ocn, torch, lay))
             del lay
