@@ -537,7 +537,9 @@ class Kernel:
         """Y = A^T M A per accumulator element (order of src/store_and_transform_output_optSTS64.cuh:29-51)
         and the 64 stores of the tile; `through` = write past the caches (a partial tile that a
         workgroup on another XCD will read)."""
-        pol = " sc0 sc1" if through else ""
+        # final outputs are written once and never read again by this kernel: non-temporal, so that
+        # they do not push the input patches that neighbouring tiles share out of L2
+        pol = " sc0 sc1" if through else " nt"
         ry = self.S["RsrcY"]
         self.row_start()
         # the last MFMAs must have written the accumulators before they are read
