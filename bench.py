@@ -41,11 +41,11 @@ DEFAULT_WORKLOAD = "resnet_n64_c64_h56_k64"
 # HBM bytes per launch of the fused kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # (profiles/), or None where not measured yet.
 MEASURED_TRAFFIC_BYTES = {
-    "resnet_n64_c64_h56_k64": 215.6e6,
-    "resnet_n128_c128_h28_k128": 261.3e6,
-    "deep_n128_c256_h14_k256": 250.1e6,
+    "resnet_n64_c64_h56_k64": 214.3e6,
+    "resnet_n128_c128_h28_k128": 261.2e6,
+    "deep_n128_c256_h14_k256": 249.7e6,
     "deep_n128_c512_h7_k512": 112.7e6,
-    "reduced_n128_c256_h14_k256_f16": 165.5e6,
+    "reduced_n128_c256_h14_k256_f16": 164.1e6,
 }
 
 
