@@ -160,10 +160,11 @@ def miopen_column(torch, lay, warmup=10, iters=200, settle_ms=150.0):
     return ev[0].elapsed_time(ev[1]) / iters
 
 
-def timeline_summary(ocn, torch, lay, launches=20, operands="f32"):
+def timeline_summary(ocn, torch, lay, launches=20, operands="f32", settle_ms=150.0):
     """Where a launch of the assembly kernels spends its time: per-workgroup stamps (kernel start,
     end of the prologue, before / after every output transform) of the last of `launches`
-    back-to-back launches with pre-transformed filters, summarised in microseconds."""
+    back-to-back launches with pre-transformed filters that follow `settle_ms` of untimed ones,
+    summarised in microseconds."""
     import numpy as np
 
     o = lay
@@ -171,6 +172,11 @@ def timeline_summary(ocn, torch, lay, launches=20, operands="f32"):
     try:
         ocn.set_operand_precision({"f32": ocn.F32, "f16": ocn.F16, "bf16": ocn.BF16}[operands])
         ocn.filter_transform(o.w, o.ws, o.K, o.C, ocn.FILTER_CRSK, ocn.WW_MFMA)
+        t_end = time.perf_counter() + settle_ms * 1e-3  # the sustained state, as for every timed region
+        while time.perf_counter() < t_end:
+            for _ in range(200):
+                ocn.conv_forward_pretransformed(o.x, o.ws, o.y, o.N, o.C, o.H, o.H, o.K)
+            torch.cuda.synchronize()
         ocn.set_timeline_buffer(buf)
         for _ in range(launches):
             ocn.conv_forward_pretransformed(o.x, o.ws, o.y, o.N, o.C, o.H, o.H, o.K)
