@@ -158,9 +158,10 @@ int opencnn_set_kernel_variant(int variant);
  * 3.06 rounds, which plain launching rounds up to 4), one persistent workgroup per CU takes an
  * equal share of (tile, 8-channel chunk) units; a tile whose channel range ends up split
  * between two workgroups is merged through the output tensor and two words of library-owned
- * device state per wave.  Results stay independent of timing (two addends commute).  Calls
- * that overlap in time on one GPU (different streams) must not both use it: pass 0 to turn it
- * off.  No counterpart in the reference, whose grid is one block per tile
+ * device state per wave.  Results stay independent of timing (two addends commute).  That
+ * state exists once per stream for the first eight streams that launch (calls on different
+ * streams may overlap in time); calls on further streams run without the split.  Pass 0 to
+ * turn it off altogether.  No counterpart in the reference, whose grid is one block per tile
  * (src/convolutionForward_32x64x8.cu:281).
  */
 int opencnn_set_balanced_split(int enable);

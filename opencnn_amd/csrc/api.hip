@@ -50,7 +50,7 @@ struct AsmKernels {
   hipModule_t module = nullptr, module_h16 = nullptr;
   hipFunction_t kw2 = nullptr, kw4 = nullptr, kw2_ragged = nullptr, kw4_ragged = nullptr;
   hipFunction_t f16_kw4 = nullptr, bf16_kw4 = nullptr;
-  unsigned* split_sync = nullptr;  // device address of g_split_sync on this device
+  unsigned* split_sync = nullptr;  // device address of g_split_sync (all sets) on this device
   bool ready = false;
 };
 
@@ -79,6 +79,29 @@ int asm_kernels(const AsmKernels** out) {
     k.ready = true;
   }
   *out = &k;
+  return 0;
+}
+
+// The split-merge flags come in kSyncSets sets; every stream that launches gets a set of its own
+// for the life of the process, so launches that overlap in time (different streams) never share
+// flags, and launches on one stream are ordered anyway.  *sync stays null for a stream beyond
+// the kSyncSets-th: its launches then do without the split.
+int split_state(hipStream_t st, unsigned** sync) {
+  static hipStream_t owner[opencnn::kSyncSets];
+  static int used = 0;
+  static std::mutex mu;
+  *sync = nullptr;
+  const AsmKernels* ak = nullptr;
+  if (int e = asm_kernels(&ak)) return e;
+  std::lock_guard<std::mutex> lock(mu);
+  int set = -1;
+  for (int i = 0; i < used; ++i)
+    if (owner[i] == st) set = i;
+  if (set < 0 && used < opencnn::kSyncSets) {
+    owner[used] = st;
+    set = used++;
+  }
+  if (set >= 0) *sync = ak->split_sync + (size_t)set * opencnn::kSyncWords;
   return 0;
 }
 
@@ -239,7 +262,7 @@ int asm_grid(const opencnn::ConvArgs& a, int kw, int chunks, int* grid) {
   if (a.nblocks < cus)
     *grid = a.nblocks;  // one tile per workgroup
   else if (cus % 8 == 0 && cus <= opencnn::kMaxBalancedBlocks &&
-           (a.nblocks % cus == 0 || g_balance.load() != 0))
+           (a.nblocks % cus == 0 || (g_balance.load() != 0 && a.sync != nullptr)))
     *grid = cus;
   return 0;
 }
@@ -269,7 +292,7 @@ int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmKernels* ak, const As
   ka.x = a.x;
   ka.usw = a.usw;
   ka.y = a.y;
-  ka.sync = ak->split_sync;
+  ka.sync = a.sync;
   ka.N = a.N;
   ka.H = a.H;
   ka.W = a.W;
@@ -398,7 +421,7 @@ int launch_hip(const opencnn::ConvArgs& a, int kw, bool ragged, bool allow_strea
   // the chunk-units split evenly (every tile then has at most two contributors).
   int cus = 0;
   if (int e = compute_units(&cus)) return e;
-  const bool balanced = g_balance.load() != 0 && a.nblocks > cus && a.nblocks % cus != 0 &&
+  const bool balanced = g_balance.load() != 0 && a.sync != nullptr && a.nblocks > cus && a.nblocks % cus != 0 &&
                         cus % 8 == 0 && cus <= opencnn::kMaxBalancedBlocks &&
                         (long long)a.nblocks * (a.C / 8) <= kMaxElems;
   if (balanced) grid = dim3(cus);
@@ -443,6 +466,7 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   a.colgroups = a.tiles_h * a.tiles_w * a.ngroups;
   a.kgroups = (filt_k + 31) / 32;
   a.nblocks = a.colblocks = 0;
+  if (int e = split_state(st, &a.sync)) return e;
   const int precision = g_precision.load();
   if (precision != OPENCNN_F32) {
     const int v = g_variant.load();

@@ -45,6 +45,7 @@ struct ConvArgs {
   int colgroups;         // tiles_h * tiles_w * ngroups   (wave-level column tiles)
   int kgroups;           // ceil(K / 32)
   int nblocks;           // workgroup tiles: filter blocks x column blocks
+  unsigned* sync;        // split-merge flags of this launch's stream (one set of g_split_sync)
   int colblocks;         // column blocks; workgroup tile T = filter block T / colblocks,
                          // column block T % colblocks (LDS kernels): an XCD's contiguous
                          // range of tiles then needs one filter block's share of Ww, which
@@ -347,9 +348,12 @@ __global__ void __launch_bounds__(256) wino_f32_fused(ConvArgs a) {
 // so the result does not depend on the arrival order.  The second wave only ever waits for a
 // wave that is already running its epilogue, never for one that has yet to be scheduled.
 constexpr int kMaxBalancedBlocks = 1024;
-// [boundary between workgroups b and b+1][wave] -> {ticket, flag}; zero between launches
-// (the second contributor clears its pair).  Launches that overlap on one GPU would share it.
-static __device__ unsigned g_split_sync[kMaxBalancedBlocks * 4 * 2];
+// [set][boundary between workgroups b and b+1][wave] -> {ticket, flag}; zero between launches
+// (the second contributor clears its pair).  Launches that overlap in time must not share a
+// set: the host hands every stream its own (kSyncSets streams at most, see api.hip).
+constexpr int kSyncSets = 8;
+constexpr int kSyncWords = kMaxBalancedBlocks * 4 * 2;
+static __device__ unsigned g_split_sync[kSyncSets * kSyncWords];
 
 template <int KW, bool BALANCED, bool RAGGED = false>
 __global__ void __launch_bounds__(256) wino_f32_fused_lds(ConvArgs a) {
@@ -473,7 +477,7 @@ __global__ void __launch_bounds__(256) wino_f32_fused_lds(ConvArgs a) {
     // All traffic of the hand-over (partial result, ticket, flag) goes straight to memory with
     // per-access system-scope policy; no fence is used, because a device-scope fence writes
     // back / invalidates the whole L2 of the XCD under the other 31 workgroups' feet.
-    unsigned* sync = g_split_sync + ((c0 > 0 ? L - 1 : L) * 4 + wave) * 2;
+    unsigned* sync = a.sync + ((c0 > 0 ? L - 1 : L) * 4 + wave) * 2;
     unsigned ticket = 0;
     if (lane == 0) ticket = __hip_atomic_fetch_add(sync, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     ticket = __builtin_amdgcn_readfirstlane(ticket);
@@ -750,12 +754,12 @@ __global__ void __launch_bounds__(256) wino_f32_stream(ConvArgs a) {
         // other part of that tile is the LAST segment of the previous workgroup, finishes late
         // and merges.  (Ranges are at least one tile long, so a segment is never both.)
         if (seg_first > 0) {
-          unsigned* flag = g_split_sync + ((L - 1) * 4 + wave) * 2 + 1;
+          unsigned* flag = a.sync + ((L - 1) * 4 + wave) * 2 + 1;
           store_tile<kStorePublish>(a, w, acc);
           asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // write-through stores acknowledged
           if (lane == 0) __hip_atomic_store(flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         } else {
-          unsigned* flag = g_split_sync + (L * 4 + wave) * 2 + 1;
+          unsigned* flag = a.sync + (L * 4 + wave) * 2 + 1;
           // normally set long ago; bounded wait all the same (never hang the GPU on a bug)
           for (int spin = 0; spin < (1 << 22); ++spin) {
             if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0) break;

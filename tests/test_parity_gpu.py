@@ -598,6 +598,40 @@ def test_non_default_stream(ocn, oracle, torch_gpu):
     check_against_oracle(oracle, y, x, w)
 
 
+def test_layers_on_different_streams_may_overlap(ocn, oracle, torch_gpu):
+    # two layers whose tiles are cut between workgroups (784 and 800 tiles on 256 CUs), launched
+    # back to back on two streams without synchronisation in between, so that they may run at the
+    # same time: every stream has split-merge flags of its own, the results are the serial ones.
+    # Ten streams in all: more than the library has flag sets for (the extra ones run unsplit).
+    print("overlapping streams", flush=True)
+    torch = torch_gpu
+    shapes = [(64, 32, 56, 56, 64), (64, 32, 40, 40, 128)]
+    runners, want = [], []
+    for N, C, H, W, K in shapes:
+        x, w = make_tensors(ocn, N, C, H, W, K)
+        r = Runner(ocn, torch, x, w)
+        want.append(r.split())
+        runners.append(r)
+    streams = [torch.cuda.Stream() for _ in range(10)]
+    torch.cuda.synchronize()
+    try:
+        for rep in range(5):
+            for r in runners:
+                r.raw.fill_(float("nan"))
+            torch.cuda.synchronize()
+            for i, r in enumerate(runners):
+                ocn.set_stream(streams[(2 * rep + i) % len(streams)])
+                ocn.conv_forward_pretransformed(r.xd, r.ws, r.yd, r.N, r.C, r.H, r.W, r.K)
+            torch.cuda.synchronize()
+            for r, y in zip(runners, want):
+                # not bit for bit: a stream without flags of its own runs the unsplit launch, which
+                # associates the channel sum differently; a lost or foreign partial tile is far off
+                rel, _, _ = oracle.compare(r.result(), y)
+                assert rel <= 1e-6, f"rep {rep}: rel-L2 against the serial result {rel:.3e}"
+    finally:
+        ocn.set_stream(None)
+
+
 def test_random_shapes_on_every_kernel_family(ocn, oracle, torch_gpu):
     # seeded sweep over batch sizes, channel and filter counts inside and outside the reference's
     # tiling, square and rectangular images, default / HIP-only kernels, balanced split on / off:
