@@ -4,10 +4,10 @@
  * Plain C: pointers and sizes only.  Every device pointer is memory the CALLER
  * allocated on the current HIP device; the library allocates no tensors or workspaces.  Its
  * state between calls is the process-wide settings of the opencnn_set_* calls below (stream,
- * kernel variant, balanced split, operand precision), the code object of its assembly kernels
+ * kernel variant, balanced split, operand precision), the code objects of its assembly kernels
  * (embedded in the library, loaded once per device by opencnn_init or the first launch) and
- * 8 KB of static device memory that the balanced split uses to hand tiles over between
- * workgroups (zero between launches).
+ * 256 KB of static device memory that the balanced split uses to hand tiles over between
+ * workgroups (eight sets of flags, one per stream; zero between launches).
  * All entry points return a hipError_t value as int (0 == hipSuccess); launches are
  * asynchronous on the selected stream, exactly like the reference, which returns
  * cudaGetLastError() right after its two launches
