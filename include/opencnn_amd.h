@@ -51,8 +51,9 @@ enum {
  * GEMM operand precision of later calls (default OPENCNN_F32, the reference's only mode).
  * With OPENCNN_F16 / OPENCNN_BF16 both transforms and the accumulation stay fp32, but the
  * transformed input and the transformed filter are rounded to nearest-even once and the 16
- * batched GEMMs run on fp16 / bf16 MFMA.  Ww then holds 2-byte elements (half of the buffer
- * is used).  Needs in_c % 16 == 0 and filt_k % 64 == 0.  Tensors in HBM stay fp32.
+ * batched GEMMs run on fp16 / bf16 MFMA.  Ww then holds 2-byte elements, padded to 64 filters
+ * and 16 channels (opencnn_workspace_bytes covers both precisions).  Any in_n, in_c, filt_k.
+ * Tensors in HBM stay fp32.
  * opencnn_filter_transform(..., OPENCNN_WW_MFMA) and the fused kernel must run under the same
  * setting.
  */

@@ -142,6 +142,9 @@ constexpr long long kMaxElems = (1LL << 31) - 1;
 // Filters / channels the transformed filter is padded to (whole MFMA groups and chunks).
 long long padded_k(int filt_k) { return ((long long)filt_k + 31) / 32 * 32; }
 long long padded_c(int filt_c) { return ((long long)filt_c + 7) / 8 * 8; }
+// The same for fp16 / bf16 operands: pairs of filter groups, 16-channel chunks, 2-byte elements.
+long long padded_k_h16(int filt_k) { return ((long long)filt_k + 63) / 64 * 64; }
+long long padded_c_h16(int filt_c) { return ((long long)filt_c + 15) / 16 * 16; }
 
 // Shapes the reference takes (its BN = 32, BK = 64 halves, BC = 8 tiling); the others run on
 // rounded-up groups with predicated lanes.
@@ -152,6 +155,7 @@ bool ragged_shape(int in_n, int in_c, int filt_k) {
 int check_filter_shape(int filt_k, int filt_c) {
   REQUIRE(filt_k > 0 && filt_c > 0);
   REQUIRE(padded_k(filt_k) * padded_c(filt_c) * 16 <= kMaxElems / 4);  // Ww byte offsets stay below 2^31
+  REQUIRE(padded_k_h16(filt_k) * padded_c_h16(filt_c) * 16 <= kMaxElems / 2);
   return 0;
 }
 
@@ -173,9 +177,8 @@ int launch_fx(const float* w, float* Ww, int filt_k, int filt_c, int filter_layo
   const bool kcrs = filter_layout == OPENCNN_FILTER_KCRS;
   const int precision = g_precision.load();
   if (ww_layout == OPENCNN_WW_MFMA && precision != OPENCNN_F32) {
-    REQUIRE(filt_c % 16 == 0);
-    REQUIRE(filt_k % 32 == 0);
-    dim3 grid((filt_k + 127) / 128, filt_c / 16), block(256);
+    // padded to whole pairs of 32-wide filter groups and 16-channel chunks, zeros in the padding
+    dim3 grid((unsigned)((padded_k_h16(filt_k) + 127) / 128), (unsigned)(padded_c_h16(filt_c) / 16)), block(256);
     uint4* out = reinterpret_cast<uint4*>(Ww);
     if (precision == OPENCNN_F16) {
       if (kcrs)
@@ -215,13 +218,12 @@ int launch_transpose(const float* src, float* dst, long long rows, long long col
   return (int)hipGetLastError();
 }
 
-// fp16 / bf16 GEMM operands: 16-channel chunks, LDS kernel only.
+// fp16 / bf16 GEMM operands: 16-channel chunks, LDS kernel only; any N, C, K (RAGGED instantiations).
 int launch_h16(opencnn::ConvArgs a, int precision, hipStream_t st) {
-  REQUIRE(a.N % 32 == 0);
-  REQUIRE(a.C % 16 == 0);
-  REQUIRE(a.K % 64 == 0);
   REQUIRE((long long)a.N * a.H * a.W * 4 * 4 <= kMaxElems);  // four-channel window in bytes
-  const int kw = a.K % 128 == 0 ? 4 : 2, cw = 4 / kw;
+  const bool ragged = a.N % 32 != 0 || a.C % 16 != 0 || a.K % 64 != 0;
+  a.kgroups = (int)(padded_k_h16(a.K) / 32);  // whole pairs of filter groups
+  const int kw = a.kgroups % 4 == 0 ? 4 : 2, cw = 4 / kw;
   const long long colblocks = (a.colgroups + cw - 1) / cw;
   const long long nblocks = colblocks * (a.kgroups / kw);
   REQUIRE(nblocks <= kMaxElems / 8);
@@ -230,22 +232,21 @@ int launch_h16(opencnn::ConvArgs a, int precision, hipStream_t st) {
   dim3 grid(((a.nblocks + 7) / 8) * 8), block(256);
   const size_t lds = (size_t)cw * 3 * 16 * 2 * 4 * 32 * sizeof(unsigned);
   const bool bf = precision == OPENCNN_BF16;
-  if (kw == 4) {
-    if (bf)
-      opencnn::wino_h16_fused_lds<4, true><<<grid, block, lds, st>>>(a);
-    else
-      opencnn::wino_h16_fused_lds<4, false><<<grid, block, lds, st>>>(a);
-  } else {
+  typedef void (*Kernel)(opencnn::ConvArgs);
+  // [kw == 2][bf16][ragged]
+  static const Kernel kernels[2][2][2] = {
+      {{&opencnn::wino_h16_fused_lds<4, false, false>, &opencnn::wino_h16_fused_lds<4, false, true>},
+       {&opencnn::wino_h16_fused_lds<4, true, false>, &opencnn::wino_h16_fused_lds<4, true, true>}},
+      {{&opencnn::wino_h16_fused_lds<2, false, false>, &opencnn::wino_h16_fused_lds<2, false, true>},
+       {&opencnn::wino_h16_fused_lds<2, true, false>, &opencnn::wino_h16_fused_lds<2, true, true>}}};
+  const Kernel fn = kernels[kw == 2][bf][ragged];
+  if (kw == 2) {
     // 96 KB of LDS: above the 64 KB a kernel gets without asking (gfx950 has 160 KB per CU)
-    const void* fn = bf ? reinterpret_cast<const void*>(&opencnn::wino_h16_fused_lds<2, true>)
-                        : reinterpret_cast<const void*>(&opencnn::wino_h16_fused_lds<2, false>);
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
-    if (bf)
-      opencnn::wino_h16_fused_lds<2, true><<<grid, block, lds, st>>>(a);
-    else
-      opencnn::wino_h16_fused_lds<2, false><<<grid, block, lds, st>>>(a);
   }
+  fn<<<grid, block, lds, st>>>(a);
   return (int)hipGetLastError();
 }
 
@@ -532,7 +533,10 @@ int opencnn_tiles_dim(int in_w) {
 
 size_t opencnn_workspace_bytes(int filt_c, int filt_k) {
   if (filt_c <= 0 || filt_k <= 0) return 0;
-  return (size_t)padded_c(filt_c) * (size_t)padded_k(filt_k) * 16 * sizeof(float);
+  // enough for either operand precision (the 2-byte layout pads further: 64 filters, 16 channels)
+  const size_t f32 = (size_t)padded_c(filt_c) * (size_t)padded_k(filt_k) * 16 * sizeof(float);
+  const size_t h16 = (size_t)padded_c_h16(filt_c) * (size_t)padded_k_h16(filt_k) * 16 * 2;
+  return f32 > h16 ? f32 : h16;
 }
 
 int opencnn_set_stream(void* stream) {

@@ -53,7 +53,13 @@ __device__ __forceinline__ v16f mfma16(v4u32 a, v4u32 b, v16f c) {
 //   end of chunk i   workgroup barrier, publishing chunk i+2's V.
 // Chunk i+1's V was published by the barrier that ended chunk i-1, so the rolling reads need
 // no further synchronisation; three LDS buffers keep the writes of chunk i+2 away from them.
-template <int KW, bool BF16>
+//
+// RAGGED = shapes outside N % 32 == 0, C % 16 == 0, K % 64 == 0, handled as in the fp32 kernels:
+// groups and chunks rounded up (a.kgroups counts whole pairs of filter groups), lanes whose
+// batch element does not exist read zeros and store nothing, the four-channel window of the
+// last chunk ends with the tensor, filters and channels past K / C are zeros in the
+// transformed filter, rows past K are not stored.
+template <int KW, bool BF16, bool RAGGED = false>
 __global__ void __launch_bounds__(256) wino_h16_fused_lds(ConvArgs a) {
   constexpr int CW = 4 / KW;
   constexpr int SPW = 4 / KW;  // channel-quads (slots) of a chunk transformed by one wave
@@ -70,7 +76,7 @@ __global__ void __launch_bounds__(256) wino_h16_fused_lds(ConvArgs a) {
   // the last real one (they must take part in the barriers) and drops their stores.
   const int cg = live ? cg_raw : a.colgroups - 1;
   WaveTile w;
-  decode_tile(a, (L / a.colblocks) * KW + kw, cg, lane, w);
+  decode_tile<RAGGED>(a, (L / a.colblocks) * KW + kw, cg, lane, w);
   const int nl = lane & 31, j = lane >> 5;
   const size_t HWN = (size_t)a.H * a.W * a.N;
 
@@ -100,8 +106,8 @@ __global__ void __launch_bounds__(256) wino_h16_fused_lds(ConvArgs a) {
   v4u32 v[16];          // B operands, rolling one chunk ahead
   float d[SPW][2][16];  // this lane's patches (a channel pair per slot), in flight
 
-  const int chunks = a.C >> 4;
-  const unsigned u_bytes = (unsigned)((size_t)a.C * 16 * a.K * 2);
+  const int chunks = RAGGED ? (a.C + 15) >> 4 : a.C >> 4;
+  const unsigned u_bytes = (unsigned)((size_t)chunks * 16 * 16 * (a.kgroups * 32) * 2);
   auto load_u1 = [&](int p, int chunk) {
     // past the last chunk: an empty descriptor, the load returns zeros without touching memory
     const __amdgpu_buffer_rsrc_t ru = make_rsrc(a.usw, chunk < chunks ? u_bytes : 0u);
@@ -113,7 +119,9 @@ __global__ void __launch_bounds__(256) wino_h16_fused_lds(ConvArgs a) {
 #pragma unroll
     for (int s = 0; s < SPW; ++s) {
       const int c0 = __builtin_amdgcn_readfirstlane(16 * ch + 4 * (kw * SPW + s));
-      const __amdgpu_buffer_rsrc_t r = make_rsrc(a.x + (size_t)c0 * HWN, (unsigned)(4 * HWN * sizeof(float)));
+      int window = 4;  // channels behind the descriptor
+      if (RAGGED) window = a.C - c0 < 0 ? 0 : (a.C - c0 < 4 ? a.C - c0 : 4);
+      const __amdgpu_buffer_rsrc_t r = make_rsrc(a.x + (size_t)c0 * HWN, (unsigned)(window * HWN * sizeof(float)));
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         d[s][0][e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff[e], 0, 0));
@@ -171,7 +179,7 @@ __global__ void __launch_bounds__(256) wino_h16_fused_lds(ConvArgs a) {
     b1 = b2;
     b2 = b0;
   }
-  if (live) store_tile<kStorePlain>(a, w, acc);
+  if (live) store_tile<kStorePlain, RAGGED>(a, w, acc);
 }
 
 }  // namespace opencnn

@@ -105,7 +105,9 @@ __global__ void __launch_bounds__(256) fx_mfma_layout(const float* __restrict__ 
 // so that lane (h*32 + k32) of a wave fetches, with one 16-byte load per position p, the A
 // operand of one v_mfma_f32_32x32x16_{f16,bf16} (16 input channels).  U is computed in fp32 in
 // the reference's order and rounded to nearest-even once.  Thread = (k, chunk, h).
-// grid (ceil(K/128), C/16), block 256 = 2 h x 128 k.
+// grid (ceil(Kpad/128), ceil(C/16)), block 256 = 2 h x 128 k.  The layout covers
+// Kpad = 64*ceil(K/64) filters (whole pairs of 32-wide groups, the smallest workgroup of the
+// fused kernel) and 16*ceil(C/16) channels; filters / channels that do not exist are zeros.
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 typedef __bf16 v2b __attribute__((ext_vector_type(2)));
 typedef float v2fx __attribute__((ext_vector_type(2)));
@@ -123,16 +125,22 @@ __global__ void __launch_bounds__(256) fx_mfma_layout_h16(const float* __restric
   const int h = threadIdx.x >> 7;
   const int k = blockIdx.x * 128 + (threadIdx.x & 127);
   const int chunk = blockIdx.y;
-  if (k >= K) return;
+  if (k >= ((K + 63) & ~63)) return;
   float U[8][16];
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    float g[9];
-    load_filter<KCRS>(w, 16 * chunk + 8 * h + e, k, C, K, g);
-    fx_one(g, U[e]);
+    const int c = 16 * chunk + 8 * h + e;
+    if (k < K && c < C) {
+      float g[9];
+      load_filter<KCRS>(w, c, k, C, K, g);
+      fx_one(g, U[e]);
+    } else {
+#pragma unroll
+      for (int p = 0; p < 16; ++p) U[e][p] = 0.0f;
+    }
   }
   const int kg = k >> 5, k32 = k & 31;
-  uint4* o = Uh + (((size_t)kg * (C >> 4) + chunk) * 16) * 64 + h * 32 + k32;
+  uint4* o = Uh + (((size_t)kg * gridDim.y + chunk) * 16) * 64 + h * 32 + k32;
 #pragma unroll
   for (int p = 0; p < 16; ++p)
     o[(size_t)p * 64] = make_uint4(pack_pair<BF16>(U[0][p], U[1][p]), pack_pair<BF16>(U[2][p], U[3][p]),

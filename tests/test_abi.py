@@ -30,9 +30,11 @@ def test_tiles_dim_and_workspace(ocn, oracle):
         assert ocn.tiles_dim(w) == oracle.tiles_dim(w) == (w + 1) // 2
     assert ocn.workspace_bytes(256, 256) == 256 * 256 * 16 * 4
     assert ocn.workspace_bytes(0, 64) == 0
-    # shapes outside the reference's tiling: filters padded to 32, channels to 8
+    # shapes outside the reference's tiling: filters padded to 32, channels to 8 (fp32 operands)
+    # or to 64 and 16 (2-byte operands), whichever needs more
     assert ocn.workspace_bytes(12, 48) == 16 * 64 * 16 * 4
-    assert ocn.workspace_bytes(1, 1) == 8 * 32 * 16 * 4
+    assert ocn.workspace_bytes(1, 1) == max(8 * 32 * 16 * 4, 16 * 64 * 16 * 2)
+    assert ocn.workspace_bytes(24, 65) == 24 * 96 * 16 * 4
 
 
 def _call(ocn, **over):

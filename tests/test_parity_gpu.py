@@ -107,7 +107,8 @@ def test_fx_bit_exact(ocn, oracle, torch_gpu, C, K):
         out = torch.full((ocn.workspace_bytes(C, K) // 4,), float("nan"), device="cuda")
         ocn.filter_transform(wd, out, K, C, layout, ocn.WW_MFMA)
         torch.cuda.synchronize()
-        got = out.cpu().numpy()
+        used = (-(-K // 32) * 32) * (-(-C // 8) * 8) * 16  # the workspace also fits the 2-byte layout
+        got = out.cpu().numpy()[:used]
         assert np.array_equal(ocn.unswizzle_ww(got, C, K), want)
         assert not np.isnan(got).any()
         assert np.count_nonzero(got) == np.count_nonzero(want)
@@ -572,15 +573,32 @@ def test_reduced_precision_assembly_variant_rejects_other_shapes(ocn, torch_gpu)
         ocn.set_operand_precision(ocn.F32)
 
 
-def test_reduced_precision_rejects_unsupported_shapes(ocn, torch_gpu):
-    x, w = make_tensors(ocn, 32, 8, 6, 6, 64)  # C % 16 != 0
-    r = Runner(ocn, torch_gpu, x, w)
+@pytest.mark.parametrize("prec", ["f16", "bf16"])
+@pytest.mark.parametrize("N,C,H,K", [
+    (32, 8, 6, 64),     # half a 16-channel chunk
+    (33, 5, 7, 40),     # nothing divides: batch, channels, filters, odd image
+    (100, 40, 9, 250),  # two and a half chunks, four filter groups of which the last holds 26
+    (1, 1, 4, 1),       # the smallest layer
+    (48, 72, 12, 160),  # whole groups, but five of them and 4.5 chunks
+])
+def test_reduced_precision_on_shapes_outside_the_tiling(ocn, oracle, torch_gpu, prec, N, C, H, K):
+    # batch, channel and filter counts that are no multiples of 32 / 16 / 64: rounded-up groups
+    # with predicated lanes, zero padding in the transformed filter, as for fp32 operands
+    print(f"reduced ragged {prec} N={N} C={C} H={H} K={K}", flush=True)
+    x, w = make_tensors(ocn, N, C, H, H, K)
     try:
-        ocn.set_operand_precision(ocn.F16)
-        with pytest.raises(ocn.OpenCNNError):
-            r.dropin()
+        ocn.set_operand_precision(ocn.F16 if prec == "f16" else ocn.BF16)
+        r = Runner(ocn, torch_gpu, x, w)
+        y = r.dropin()
+        y2 = r.dropin()
     finally:
         ocn.set_operand_precision(ocn.F32)
+    assert not np.isnan(y).any(), "an output element was never written"
+    assert np.array_equal(y, y2)
+    rel, _, _ = oracle.compare(y, oracle.winograd_f32(x, w, 1 if prec == "f16" else 2))
+    assert rel <= REL_L2_QUANTISED_RESTATEMENT, f"rel-L2 vs quantised restatement {rel:.3e}"
+    rel64, _, _ = oracle.compare(y, oracle.direct_conv_f64(x, w))
+    assert rel64 <= REL_L2_DIRECT_REDUCED[prec], f"rel-L2 vs fp64 direct {rel64:.3e}"
 
 
 def test_non_default_stream(ocn, oracle, torch_gpu):
