@@ -284,6 +284,7 @@ struct AsmLaunch {
   int lockstep_log2 = -1;
   // fp16 / bf16 kernels (>= 0): cost of an output transform in half units; ranges are then cut on
   // a weighted line, a tile = 2 * chunks + this, and the kernel maps positions back to units.
+  int filter_groups = -1;  // fp16 / bf16 kernels: filter groups of 32 that exist
   int epilogue_half_units = -1;
 };
 
@@ -302,7 +303,7 @@ int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmKernels* ak, const As
   ka.ngroups = a.ngroups;
   ka.colgroups = a.colgroups;
   ka.colblocks = l.tile_split;
-  ka.Q = chunks * 2;
+  ka.Q = l.filter_groups >= 0 ? l.filter_groups : chunks * 2;
   ka.HWN4 = a.N * a.H * a.W * 4;
   ka.c_real = l.c_real_or_mode;
   ka.k_real = a.K;
@@ -359,9 +360,11 @@ constexpr int kEpilogueHalfUnits = 3;
 
 int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* launched) {
   *launched = false;
-  if (a.N % 32 != 0 || a.C % 16 != 0 || a.K % 128 != 0) return 0;
+  // K % 128 == 64: two waves of the last filter block have no filters; they help with the input
+  // transform, multiply zeros and store nothing.
+  if (a.N % 32 != 0 || a.C % 16 != 0 || a.K % 64 != 0) return 0;
   if ((long long)a.N * a.H * a.W * 4 * 4 > kMaxElems) return 0;  // four-channel slab in bytes
-  const int kblocks = a.kgroups / 4, chunks = a.C / 16;
+  const int kblocks = (a.kgroups + 3) / 4, chunks = a.C / 16;
   const long long nblocks = (long long)a.colgroups * kblocks;
   const long long usw_bytes = (long long)a.C * 16 * a.K * 2;
   if (nblocks > kMaxElems / 8 || usw_bytes > kMaxElems) return 0;
@@ -380,6 +383,7 @@ int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* lau
   l.chunks = chunks;
   l.usw_bytes = usw_bytes;
   l.epilogue_half_units = kEpilogueHalfUnits;
+  l.filter_groups = a.K / 32;
   // How the units are dealt.  While the whole 2-byte transformed filter leaves room in an XCD's
   // 4 MB L2 and the filter blocks are a power of two that divides the grid: one line of units per
   // filter block, walked in lockstep by neighbouring workgroups (the patches the filter blocks

@@ -28,7 +28,8 @@ What differs from the fp32 kernels:
     2-byte transformed filter is small enough for all blocks to stay there too);
   * s_waitcnt counts are derived by the generator from the issue order of the loads.
 
-Eligibility (api.hip): N % 32 == 0, C % 16 == 0, K % 128 == 0.
+Eligibility (api.hip): N % 32 == 0, C % 16 == 0, K % 64 == 0 (K % 128 == 64: two waves of the
+last filter block have no filters, see filter_descriptor).
 
 Usage: gen_wino_h16_asm.py > wino_h16_asm.s
 """
@@ -152,6 +153,7 @@ class KernelH16(Kernel):
             self.filter_block(t(0), self.sr("Tq"))
             self.e(f"s_lshl_b32 {t(0)}, {t(0)}, 2")
             self.e(f"s_add_u32 {self.sr('KgQ')}, {t(0)}, {self.sr('Kw')}")
+            self.filter_descriptor(self.sr("KgQ"))
         self.advance_cursor(self.sr("Tq"), self.sr("Cq"), 1, "q", switch)
 
     def unit_range(self, owner):
@@ -195,6 +197,30 @@ class KernelH16(Kernel):
         e(f"s_cmp_eq_u32 {self.sr('Cm')}, {self.sr('Chunks')}")
         e(f"s_cselect_b32 {self.sr('Cm')}, 0, {self.sr('Cm')}")
         e(f"s_addc_u32 {self.sr('Tm')}, {self.sr('Tm')}, 0")
+
+    # ------------------------------------------------------------------ filter groups that do not exist
+    # K % 128 == 64: the last filter block has two filter groups only.  Its other two waves still
+    # share the input transform of the column tile; they multiply zeros (their filter descriptor
+    # is empty, so their loads touch no memory) and store nothing.  The argument slot Q (twice
+    # the chunks per tile in the fp32 kernels) carries the number of real filter groups here.
+    def u_offset(self, dst, kg, c, second):
+        t = self.t
+        self.e(f"s_mul_i32 {t(0)}, {kg}, {self.sr('Chunks')}")
+        self.e(f"s_add_u32 {t(0)}, {t(0)}, {c}")
+        self.e(f"s_lshl_b32 {dst}, {t(0)}, 14")
+
+    def filter_descriptor(self, kg):
+        """RsrcU covers the transformed filter, or nothing when filter group kg does not exist."""
+        self.e(f"s_cmp_lt_u32 {kg}, {self.sr('Q')}")
+        self.e(f"s_cselect_b32 {s(self.S['RsrcU'] + 2)}, {self.sr('UswBytes')}, 0")
+
+    def m_tile_setup(self):
+        t = self.t
+        self.e(f"s_lshl_b32 {t(0)}, {self.sr('Dkb')}, 2")
+        self.e(f"s_add_u32 {t(0)}, {t(0)}, {self.sr('Kw')}")
+        self.e(f"s_cmp_lt_u32 {t(0)}, {self.sr('Q')}")
+        self.e(f"s_cselect_b32 {self.sr('Dlive')}, {self.sr('Dlive')}, 0")
+        super().m_tile_setup()
 
     def range_owner(self):
         t = self.t
@@ -453,6 +479,7 @@ class KernelH16(Kernel):
         self.decode(self.sr("Tm"))
         self.m_tile_setup()
         e(f"s_mov_b32 {self.sr('KgQ')}, {self.sr('KgM')}")
+        self.filter_descriptor(self.sr("KgQ"))
         self.patch_offsets()
         self.u_offset(self.sr("UoffQ"), self.sr("KgM"), self.sr("Cm"), False)
         self.slab_descriptor(0)

@@ -519,13 +519,15 @@ def test_reduced_precision_operands(ocn, oracle, torch_gpu, prec, N, C, H, K, xr
     print(f"  rel-L2 vs quantised restatement {rel:.2e}, vs fp64 direct {rel64:.2e}", flush=True)
 
 
-# (N, C, H, W, K) for the hand-scheduled fp16 / bf16 kernels (K % 128 == 0, C % 16 == 0):
+# (N, C, H, W, K) for the hand-scheduled fp16 / bf16 kernels (K % 64 == 0, C % 16 == 0):
 # the benchmark configuration (two filter blocks in lockstep); one tile per workgroup; one
 # 16-channel chunk; three filter blocks and an 8 MB transformed filter (one filter-block-major
 # line of units); tiles cut between workgroups with one, two and four filter blocks; odd sizes
 H16_ASM_SHAPES = [(128, 256, 14, 14, 256), (32, 32, 6, 6, 128), (32, 16, 9, 9, 256), (64, 48, 9, 9, 384),
                   (32, 512, 5, 5, 512), (64, 32, 40, 40, 128), (64, 64, 21, 21, 256), (32, 32, 30, 30, 512),
-                  (32, 32, 31, 9, 128), (96, 48, 1, 1, 128)]
+                  (32, 32, 31, 9, 128), (96, 48, 1, 1, 128),
+                  # filter counts of 64, 192 and 320: the last filter block holds two filter groups
+                  (64, 64, 56, 56, 64), (32, 32, 12, 12, 192), (32, 16, 7, 7, 64), (64, 48, 19, 19, 320)]
 
 
 @pytest.mark.parametrize("prec", ["f16", "bf16"])
@@ -559,7 +561,7 @@ def test_reduced_precision_assembly_kernels(ocn, oracle, torch_gpu, prec, N, C, 
 
 
 def test_reduced_precision_assembly_variant_rejects_other_shapes(ocn, torch_gpu):
-    x, w = make_tensors(ocn, 32, 16, 6, 6, 64)  # K % 128 != 0: the HIP kernel's shape
+    x, w = make_tensors(ocn, 32, 16, 6, 6, 96)  # K % 64 != 0: the HIP kernel's shape
     r = Runner(ocn, torch_gpu, x, w)
     try:
         ocn.set_operand_precision(ocn.F16)
