@@ -278,8 +278,8 @@ struct AsmLaunch {
   // The divisor that takes a workgroup tile index apart: the column blocks (filter-block major
   // line of units), or, with lockstep_log2 >= 0, the filter blocks.
   int tile_split = 1;
-  // fp32 kernels: the real channel count (ragged shapes).  fp16 / bf16 kernels: 0 = one line of
-  // units per filter block (2^lockstep_log2 of them, walked in lockstep), 1 = one line.
+  // The real channel count.  fp16 / bf16 kernels: positive = one line of units per filter block
+  // (2^lockstep_log2 of them, walked in lockstep), negative = one line.
   int c_real_or_mode = 0;
   int lockstep_log2 = -1;
   // fp16 / bf16 kernels (>= 0): cost of an output transform in half units; ranges are then cut on
@@ -288,7 +288,7 @@ struct AsmLaunch {
   int epilogue_half_units = -1;
 };
 
-int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmKernels* ak, const AsmLaunch& l, hipStream_t st) {
+int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmLaunch& l, hipStream_t st) {
   const int chunks = l.chunks, grid = l.grid;
   AsmKernArgs ka{};
   ka.x = a.x;
@@ -350,7 +350,7 @@ int launch_asm(const opencnn::ConvArgs& a, int kw, int grid, bool ragged, size_t
   l.usw_bytes = padded_c(a.C) * 16 * padded_k(a.K) * 4;
   l.tile_split = a.colblocks;
   l.c_real_or_mode = a.C;
-  return launch_asm_kernel(a, ak, l, st);
+  return launch_asm_kernel(a, l, st);
 }
 
 // The hand-scheduled fp16 / bf16 kernels (gen_wino_h16_asm.py) take whole 128-filter blocks and
@@ -362,11 +362,13 @@ int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* lau
   *launched = false;
   // K % 128 == 64: two waves of the last filter block have no filters; they help with the input
   // transform, multiply zeros and store nothing.
-  if (a.N % 32 != 0 || a.C % 16 != 0 || a.K % 64 != 0) return 0;
+  // Any channel count: the last chunk's missing channels read as zeros (descriptor cut at the
+  // tensor's end) and meet zero rows of the padded transformed filter.
+  if (a.N % 32 != 0 || a.K % 64 != 0) return 0;
   if ((long long)a.N * a.H * a.W * 4 * 4 > kMaxElems) return 0;  // four-channel slab in bytes
-  const int kblocks = (a.kgroups + 3) / 4, chunks = a.C / 16;
+  const int kblocks = (a.kgroups + 3) / 4, chunks = (int)(padded_c_h16(a.C) / 16);
   const long long nblocks = (long long)a.colgroups * kblocks;
-  const long long usw_bytes = (long long)a.C * 16 * a.K * 2;
+  const long long usw_bytes = padded_c_h16(a.C) * 16 * a.K * 2;
   if (nblocks > kMaxElems / 8 || usw_bytes > kMaxElems) return 0;
   if (nblocks * (2LL * chunks + kEpilogueHalfUnits) > kMaxElems) return 0;  // the weighted line of units
   a.nblocks = (int)nblocks;
@@ -392,13 +394,13 @@ int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* lau
   while ((1 << log2k) < kblocks) ++log2k;
   if (usw_bytes <= (2 << 20) && (1 << log2k) == kblocks && grid % kblocks == 0) {
     l.tile_split = kblocks;
-    l.c_real_or_mode = 0;
+    l.c_real_or_mode = a.C;
     l.lockstep_log2 = log2k;
   } else {
     l.tile_split = a.colblocks;
-    l.c_real_or_mode = 1;
+    l.c_real_or_mode = -a.C;
   }
-  const int e = launch_asm_kernel(a, ak, l, st);
+  const int e = launch_asm_kernel(a, l, st);
   *launched = e == 0;
   return e;
 }

@@ -28,8 +28,9 @@ What differs from the fp32 kernels:
     2-byte transformed filter is small enough for all blocks to stay there too);
   * s_waitcnt counts are derived by the generator from the issue order of the loads.
 
-Eligibility (api.hip): N % 32 == 0, C % 16 == 0, K % 64 == 0 (K % 128 == 64: two waves of the
-last filter block have no filters, see filter_descriptor).
+Eligibility (api.hip): N % 32 == 0, K % 64 == 0, any C (the last chunk may hold fewer than 16
+channels, see slab_descriptor; K % 128 == 64: two waves of the last filter block have no
+filters, see filter_descriptor).
 
 Usage: gen_wino_h16_asm.py > wino_h16_asm.s
 """
@@ -76,8 +77,8 @@ class KernelH16(Kernel):
         self.MP = [self.V[n] + i for n in ("T", "TA", "TB", "MPX") for i in range(16)]
 
     # ------------------------------------------------------------------ tile order
-    # Two ways to deal the units, chosen by the host through the argument slot that carries the
-    # real channel count of the ragged fp32 kernels:
+    # Two ways to deal the units, chosen by the host through the sign of the argument that carries
+    # the channel count (+C: way 0, -C: way 1):
     #   0  one line of (column block, chunk) units PER FILTER BLOCK.  The workgroups L = r*B + b
     #      (B filter blocks, a power of two; the Colblocks slot holds B, the Scb slot log2 B) own
     #      range r of filter block b: the B workgroups of a range sit on neighbouring CUs of one
@@ -222,9 +223,28 @@ class KernelH16(Kernel):
         self.e(f"s_cselect_b32 {self.sr('Dlive')}, {self.sr('Dlive')}, 0")
         super().m_tile_setup()
 
+    def slab_descriptor(self, j):
+        """RsrcX = the four-channel slab of this wave in chunk Cp, cut where the tensor ends: the
+        channels past a count that is no multiple of 16 read as zeros (the SGPR offset that selects
+        a lane's second channel takes part in the range check of the load)."""
+        t = self.t
+        rx = self.S["RsrcX"]
+        self.e(f"s_lshl_b32 {t(0)}, {self.sr('Cp')}, 2")
+        self.e(f"s_add_u32 {t(0)}, {t(0)}, {self.sr('KwSpw')}")
+        self.e(f"s_abs_i32 {t(2)}, {self.sr('Creal')}")
+        self.e(f"s_lshl_b32 {t(1)}, {t(0)}, 2")
+        self.e(f"s_sub_i32 {t(2)}, {t(2)}, {t(1)}")
+        self.e(f"s_max_i32 {t(2)}, {t(2)}, 0")
+        self.e(f"s_min_i32 {t(2)}, {t(2)}, 4")
+        self.e(f"s_mul_i32 {s(rx + 2)}, {t(2)}, {self.sr('HWN4')}")
+        self.e(f"s_mul_hi_u32 {t(1)}, {t(0)}, {self.sr('Slab')}")
+        self.e(f"s_mul_i32 {t(0)}, {t(0)}, {self.sr('Slab')}")
+        self.e(f"s_add_u32 {s(rx)}, {s(self.S['X'])}, {t(0)}")
+        self.e(f"s_addc_u32 {s(rx + 1)}, {s(self.S['X'] + 1)}, {t(1)}")
+
     def range_owner(self):
         t = self.t
-        self.e(f"s_cmp_eq_u32 {self.sr('Creal')}, 0")
+        self.e(f"s_cmp_gt_i32 {self.sr('Creal')}, 0")
         self.e(f"s_cselect_b32 {t(0)}, {self.sr('Scb')}, 0")
         self.e(f"s_lshr_b32 {self.sr('Lr')}, {self.sr('L')}, {t(0)}")
         self.e(f"s_sub_u32 {t(0)}, {self.sr('Colblocks')}, 1")
@@ -237,14 +257,14 @@ class KernelH16(Kernel):
         self.div(t(1), T, self.sr("Mcb"), self.sr("Scb"))  # meaningless in mode 0, not used there
         self.e(f"s_mul_i32 {t(0)}, {t(1)}, {self.sr('Colblocks')}")
         self.e(f"s_sub_u32 {t(0)}, {T}, {t(0)}")
-        self.e(f"s_cmp_eq_u32 {self.sr('Creal')}, 0")
+        self.e(f"s_cmp_gt_i32 {self.sr('Creal')}, 0")
         self.e(f"s_cselect_b32 {self.sr('Dkb')}, {self.sr('Kbf')}, {t(1)}")
         self.e(f"s_cselect_b32 {t(0)}, {T}, {t(0)}")
 
     def filter_block(self, dst, T):
         t = self.t
         self.div(t(1), T, self.sr("Mcb"), self.sr("Scb"))
-        self.e(f"s_cmp_eq_u32 {self.sr('Creal')}, 0")
+        self.e(f"s_cmp_gt_i32 {self.sr('Creal')}, 0")
         self.e(f"s_cselect_b32 {dst}, {self.sr('Kbf')}, {t(1)}")
 
     def flag_address(self, previous):
@@ -253,7 +273,7 @@ class KernelH16(Kernel):
         t = self.t
         fl = self.S["Fl"]
         if previous:
-            self.e(f"s_cmp_eq_u32 {self.sr('Creal')}, 0")
+            self.e(f"s_cmp_gt_i32 {self.sr('Creal')}, 0")
             self.e(f"s_cselect_b32 {t(0)}, {self.sr('Colblocks')}, 1")
             self.e(f"s_sub_u32 {t(0)}, {self.sr('L')}, {t(0)}")
         else:

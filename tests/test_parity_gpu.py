@@ -519,7 +519,7 @@ def test_reduced_precision_operands(ocn, oracle, torch_gpu, prec, N, C, H, K, xr
     print(f"  rel-L2 vs quantised restatement {rel:.2e}, vs fp64 direct {rel64:.2e}", flush=True)
 
 
-# (N, C, H, W, K) for the hand-scheduled fp16 / bf16 kernels (K % 64 == 0, C % 16 == 0):
+# (N, C, H, W, K) for the hand-scheduled fp16 / bf16 kernels (N % 32 == 0, K % 64 == 0):
 # the benchmark configuration (two filter blocks in lockstep); one tile per workgroup; one
 # 16-channel chunk; three filter blocks and an 8 MB transformed filter (one filter-block-major
 # line of units); tiles cut between workgroups with one, two and four filter blocks; odd sizes
@@ -527,7 +527,9 @@ H16_ASM_SHAPES = [(128, 256, 14, 14, 256), (32, 32, 6, 6, 128), (32, 16, 9, 9, 2
                   (32, 512, 5, 5, 512), (64, 32, 40, 40, 128), (64, 64, 21, 21, 256), (32, 32, 30, 30, 512),
                   (32, 32, 31, 9, 128), (96, 48, 1, 1, 128),
                   # filter counts of 64, 192 and 320: the last filter block holds two filter groups
-                  (64, 64, 56, 56, 64), (32, 32, 12, 12, 192), (32, 16, 7, 7, 64), (64, 48, 19, 19, 320)]
+                  (64, 64, 56, 56, 64), (32, 32, 12, 12, 192), (32, 16, 7, 7, 64), (64, 48, 19, 19, 320),
+                  # channel counts that are no multiple of 16 (an RGB first layer; odd; one over a chunk)
+                  (64, 3, 20, 20, 64), (32, 5, 6, 6, 64), (32, 17, 7, 7, 256), (32, 40, 9, 9, 128)]
 
 
 @pytest.mark.parametrize("prec", ["f16", "bf16"])
