@@ -114,7 +114,9 @@ struct AsmKernArgs {
   int32_t N, H, W, chunks, tiles_w, ngroups, colgroups, colblocks;
   int32_t Q, HWN4, units_q, units_rem, usw_bytes, grid_per_xcd;
   uint32_t m_chunks, s_chunks, m_colblocks, s_colblocks, m_ngroups, s_ngroups, m_tiles_w, s_tiles_w;
-  int32_t c_real, k_real;  // read by the _ragged kernels only
+  // _ragged fp32 kernels: real channel and filter counts.  fp16 / bf16 kernels: the channel count
+  // (its sign selects the unit order) and the weighted length of a tile.
+  int32_t c_real, k_real;
   long long* timeline;     // 64 entries per workgroup, or null
 };
 static_assert(sizeof(AsmKernArgs) == 136, "kernel argument block");
