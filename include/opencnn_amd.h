@@ -137,8 +137,8 @@ int opencnn_set_stream(void *stream);
  *                            units that are not a multiple of them, the balanced split switched
  *                            on); otherwise later launches return hipErrorInvalidValue.
  *                            With fp16 / bf16 operands (opencnn_set_operand_precision): units of
- *                            16 channels, shapes with in_n % 32 == 0 and filt_k % 64 == 0
- *                            (any in_c)
+ *                            16 channels, any shape (the condition on the balanced split
+ *                            stays)
  *   OPENCNN_KERNEL_HIP       the HIP C++ kernels only: the LDS variant when the 32-wide filter
  *                            groups (filt_k / 32, rounded up) pair up (as one continuous pipeline
  *                            over all tiles of a workgroup when the balanced split is in use),

@@ -286,7 +286,7 @@ struct AsmLaunch {
   int lockstep_log2 = -1;
   // fp16 / bf16 kernels (>= 0): cost of an output transform in half units; ranges are then cut on
   // a weighted line, a tile = 2 * chunks + this, and the kernel maps positions back to units.
-  int filter_groups = -1;  // fp16 / bf16 kernels: filter groups of 32 that exist
+  int filters = -1;  // fp16 / bf16 kernels: the real filter count
   int epilogue_half_units = -1;
 };
 
@@ -305,7 +305,7 @@ int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmLaunch& l, hipStream_
   ka.ngroups = a.ngroups;
   ka.colgroups = a.colgroups;
   ka.colblocks = l.tile_split;
-  ka.Q = l.filter_groups >= 0 ? l.filter_groups : chunks * 2;
+  ka.Q = l.filters >= 0 ? l.filters : chunks * 2;
   ka.HWN4 = a.N * a.H * a.W * 4;
   ka.c_real = l.c_real_or_mode;
   ka.k_real = a.K;
@@ -362,15 +362,14 @@ constexpr int kEpilogueHalfUnits = 3;
 
 int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* launched) {
   *launched = false;
-  // K % 128 == 64: two waves of the last filter block have no filters; they help with the input
-  // transform, multiply zeros and store nothing.
-  // Any channel count: the last chunk's missing channels read as zeros (descriptor cut at the
-  // tensor's end) and meet zero rows of the padded transformed filter.
-  if (a.N % 32 != 0 || a.K % 64 != 0) return 0;
+  // Any shape.  Waves of the last filter block whose 32 filters do not exist help with the input
+  // transform, multiply zeros and store nothing; the last chunk's missing channels read as zeros
+  // (descriptor cut at the tensor's end) and meet zero rows of the padded transformed filter;
+  // batch elements and filter rows that do not exist are masked per lane / per row.
   if ((long long)a.N * a.H * a.W * 4 * 4 > kMaxElems) return 0;  // four-channel slab in bytes
   const int kblocks = (a.kgroups + 3) / 4, chunks = (int)(padded_c_h16(a.C) / 16);
   const long long nblocks = (long long)a.colgroups * kblocks;
-  const long long usw_bytes = padded_c_h16(a.C) * 16 * a.K * 2;
+  const long long usw_bytes = padded_c_h16(a.C) * 16 * padded_k_h16(a.K) * 2;
   if (nblocks > kMaxElems / 8 || usw_bytes > kMaxElems) return 0;
   if (nblocks * (2LL * chunks + kEpilogueHalfUnits) > kMaxElems) return 0;  // the weighted line of units
   a.nblocks = (int)nblocks;
@@ -387,7 +386,7 @@ int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* lau
   l.chunks = chunks;
   l.usw_bytes = usw_bytes;
   l.epilogue_half_units = kEpilogueHalfUnits;
-  l.filter_groups = a.K / 32;
+  l.filters = a.K;
   // How the units are dealt.  While the whole 2-byte transformed filter leaves room in an XCD's
   // 4 MB L2 and the filter blocks are a power of two that divides the grid: one line of units per
   // filter block, walked in lockstep by neighbouring workgroups (the patches the filter blocks

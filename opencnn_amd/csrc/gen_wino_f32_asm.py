@@ -85,6 +85,8 @@ def a(i, n=1):
 
 
 class Kernel:
+    K_REAL = "Kreal"  # the scalar register with the real filter count (ragged K)
+
     def __init__(self, KW, ragged=False):
         """ragged: shapes outside N % 32 == 0, K % 32 == 0, C % 8 == 0.  Groups and chunks are
         rounded up by the host; lanes whose batch element does not exist read zeros and store
@@ -92,6 +94,8 @@ class Kernel:
         past K fall outside the row's num_records.  The inner loop is the same."""
         self.KW = KW
         self.ragged = ragged
+        # batch elements, and filters, that do not exist are masked (the fp16 / bf16 kernels always do)
+        self.ragged_n = self.ragged_k = ragged
         self.CW = 4 // KW
         self.SPW = 4 // KW
         self.lines = []
@@ -217,7 +221,7 @@ class Kernel:
         self.e(f"s_add_i32 {t(2)}, {t(2)}, {t(3)}")
         self.e(f"s_lshl_b32 {t(3)}, {self.sr('Dng')}, 7")
         self.e(f"s_add_i32 {t(2)}, {t(2)}, {t(3)}")  # byte offset of element (0,0), may be negative
-        if self.ragged:
+        if self.ragged_n:
             self.alive_lanes()
         for i in range(4):
             self.e(f"s_add_i32 {t(4)}, {t(0)}, {i}")
@@ -231,7 +235,7 @@ class Kernel:
                 self.e(f"s_cmp_lg_u32 {t(4)}, 0")
                 self.e(f"s_cselect_b32 {t(5)}, {t(3)}, 0x{OOB:x}")
                 self.e(f"v_add_u32 {self.vr('VOFF', i * 4 + j)}, {t(5)}, {self.vr('LaneX')}")
-                if self.ragged:
+                if self.ragged_n:
                     self.e(f"v_cndmask_b32 {self.vr('VOFF', i * 4 + j)}, {self.vr('Oob')}, {self.vr('VOFF', i * 4 + j)}, vcc")
                 if j < 3:
                     self.e(f"s_add_i32 {t(3)}, {t(3)}, {self.sr('ColStep')}")
@@ -290,13 +294,13 @@ class Kernel:
         self.e(f"s_cmp_lt_u32 {t(1)}, {self.sr('W')}")
         self.e(f"s_cselect_b32 {t(1)}, {self.sr('Dlive')}, 0")  # column 1 stored
         self.e(f"s_and_b32 {t(2)}, {t(0)}, {t(1)}")
-        if self.ragged:
+        if self.ragged_n:
             self.alive_lanes()
         for q, ok in enumerate([self.sr("Dlive"), t(1), t(0), t(2)]):
             self.e(f"s_cmp_lg_u32 {ok}, 0")
             self.e(f"s_cselect_b32 {t(3)}, 0, 0x{OOB:x}")
             self.e(f"v_or_b32 {self.vr('Eff', q)}, {t(3)}, {self.vr('Off', q)}")
-            if self.ragged:
+            if self.ragged_n:
                 self.e(f"v_cndmask_b32 {self.vr('Eff', q)}, {self.vr('Oob')}, {self.vr('Eff', q)}, vcc")
         # first row of the tile: y + kg*32*HWN4 + ((2ty*W + 2tx)*N + ng*32)*4
         yt = self.S["Yt"]
@@ -504,7 +508,7 @@ class Kernel:
         ry = self.S["RsrcY"]
         self.e(f"s_mov_b32 {s(ry)}, {s(self.S['Yt'])}")
         self.e(f"s_mov_b32 {s(ry + 1)}, {s(self.S['Yt'] + 1)}")
-        if self.ragged:
+        if self.ragged_k:
             self.e(f"s_lshl_b32 {self.t(2)}, {self.sr('KgM')}, 5")   # first filter of the wave tile
             self.e(f"s_lshl_b32 {self.t(3)}, {self.sr('HWN4')}, 2")  # lane offsets below this: hsel = 0
             self.row_limit(0)
@@ -515,10 +519,10 @@ class Kernel:
         t = self.t
         ry = self.S["RsrcY"]
         self.e(f"s_add_u32 {t(0)}, {t(2)}, {8 * (r >> 2) + (r & 3)}")
-        self.e(f"s_cmp_lt_u32 {t(0)}, {self.sr('Kreal')}")
+        self.e(f"s_cmp_lt_u32 {t(0)}, {self.sr(self.K_REAL)}")
         self.e(f"s_cselect_b32 {t(1)}, {t(3)}, 0")
         self.e(f"s_add_u32 {t(0)}, {t(0)}, 4")
-        self.e(f"s_cmp_lt_u32 {t(0)}, {self.sr('Kreal')}")
+        self.e(f"s_cmp_lt_u32 {t(0)}, {self.sr(self.K_REAL)}")
         self.e(f"s_cselect_b32 {s(ry + 2)}, 0x{OOB:x}, {t(1)}")
 
     def row_advance(self, r):
@@ -530,7 +534,7 @@ class Kernel:
         for _ in range(mult):
             self.e(f"s_add_u32 {s(ry)}, {s(ry)}, {self.sr('HWN4')}")
             self.e(f"s_addc_u32 {s(ry + 1)}, {s(ry + 1)}, 0")
-        if self.ragged:
+        if self.ragged_k:
             self.row_limit(r + 1)
 
     def epilogue(self, through):

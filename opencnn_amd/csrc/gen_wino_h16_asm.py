@@ -28,9 +28,10 @@ What differs from the fp32 kernels:
     2-byte transformed filter is small enough for all blocks to stay there too);
   * s_waitcnt counts are derived by the generator from the issue order of the loads.
 
-Eligibility (api.hip): N % 32 == 0, K % 64 == 0, any C (the last chunk may hold fewer than 16
-channels, see slab_descriptor; K % 128 == 64: two waves of the last filter block have no
-filters, see filter_descriptor).
+Any N, C, K (api.hip pads the transformed filter with zeros to whole chunks of 16 channels and
+pairs of 32-wide filter groups): batch elements and filter rows that do not exist are masked as
+in the _ragged fp32 kernels, the last chunk's slab ends with the tensor (slab_descriptor), waves
+of the last filter block without filters load and store nothing (filter_descriptor).
 
 Usage: gen_wino_h16_asm.py > wino_h16_asm.s
 """
@@ -51,11 +52,13 @@ class Wait:
 
 class KernelH16(Kernel):
     SLAB_CHANNELS = 4
+    K_REAL = "Q"  # the argument slot Q (twice the chunks per tile in the fp32 kernels) carries K here
 
     def __init__(self, bf16):
         self.bf16 = bf16
         self.KW, self.CW, self.SPW = 4, 1, 1
         self.ragged = False
+        self.ragged_n = self.ragged_k = True  # any N, K: a handful of scalar instructions per tile
         self.lines, self.outofline, self.nlabel = [], [], 0
         self.name = f"wino_{'bf16' if bf16 else 'f16'}_asm_kw4"
         self.alloc()
@@ -200,10 +203,11 @@ class KernelH16(Kernel):
         e(f"s_addc_u32 {self.sr('Tm')}, {self.sr('Tm')}, 0")
 
     # ------------------------------------------------------------------ filter groups that do not exist
-    # K % 128 == 64: the last filter block has two filter groups only.  Its other two waves still
-    # share the input transform of the column tile; they multiply zeros (their filter descriptor
-    # is empty, so their loads touch no memory) and store nothing.  The argument slot Q (twice
-    # the chunks per tile in the fp32 kernels) carries the number of real filter groups here.
+    # The last filter block may hold fewer than four filter groups (K <= 96 mod 128).  The waves
+    # without one still share the input transform of the column tile; they multiply zeros (their
+    # filter descriptor is empty, so their loads touch no memory) and store nothing.  A group that
+    # exists in part (K % 32 != 0) finds zero rows in the padded transformed filter and stores
+    # its real rows only (row_limit).  The argument slot Q carries K.
     def u_offset(self, dst, kg, c, second):
         t = self.t
         self.e(f"s_mul_i32 {t(0)}, {kg}, {self.sr('Chunks')}")
@@ -212,13 +216,16 @@ class KernelH16(Kernel):
 
     def filter_descriptor(self, kg):
         """RsrcU covers the transformed filter, or nothing when filter group kg does not exist."""
-        self.e(f"s_cmp_lt_u32 {kg}, {self.sr('Q')}")
+        t = self.t
+        self.e(f"s_lshl_b32 {t(3)}, {kg}, 5")
+        self.e(f"s_cmp_lt_u32 {t(3)}, {self.sr('Q')}")
         self.e(f"s_cselect_b32 {s(self.S['RsrcU'] + 2)}, {self.sr('UswBytes')}, 0")
 
     def m_tile_setup(self):
         t = self.t
         self.e(f"s_lshl_b32 {t(0)}, {self.sr('Dkb')}, 2")
         self.e(f"s_add_u32 {t(0)}, {t(0)}, {self.sr('Kw')}")
+        self.e(f"s_lshl_b32 {t(0)}, {t(0)}, 5")
         self.e(f"s_cmp_lt_u32 {t(0)}, {self.sr('Q')}")
         self.e(f"s_cselect_b32 {self.sr('Dlive')}, {self.sr('Dlive')}, 0")
         super().m_tile_setup()

@@ -519,7 +519,7 @@ def test_reduced_precision_operands(ocn, oracle, torch_gpu, prec, N, C, H, K, xr
     print(f"  rel-L2 vs quantised restatement {rel:.2e}, vs fp64 direct {rel64:.2e}", flush=True)
 
 
-# (N, C, H, W, K) for the hand-scheduled fp16 / bf16 kernels (N % 32 == 0, K % 64 == 0):
+# (N, C, H, W, K) for the hand-scheduled fp16 / bf16 kernels (any shape):
 # the benchmark configuration (two filter blocks in lockstep); one tile per workgroup; one
 # 16-channel chunk; three filter blocks and an 8 MB transformed filter (one filter-block-major
 # line of units); tiles cut between workgroups with one, two and four filter blocks; odd sizes
@@ -529,7 +529,10 @@ H16_ASM_SHAPES = [(128, 256, 14, 14, 256), (32, 32, 6, 6, 128), (32, 16, 9, 9, 2
                   # filter counts of 64, 192 and 320: the last filter block holds two filter groups
                   (64, 64, 56, 56, 64), (32, 32, 12, 12, 192), (32, 16, 7, 7, 64), (64, 48, 19, 19, 320),
                   # channel counts that are no multiple of 16 (an RGB first layer; odd; one over a chunk)
-                  (64, 3, 20, 20, 64), (32, 5, 6, 6, 64), (32, 17, 7, 7, 256), (32, 40, 9, 9, 128)]
+                  (64, 3, 20, 20, 64), (32, 5, 6, 6, 64), (32, 17, 7, 7, 256), (32, 40, 9, 9, 128),
+                  # batch sizes and filter counts outside the tiling: masked lanes and rows
+                  (33, 5, 7, 7, 40), (100, 40, 9, 9, 250), (1, 1, 4, 4, 1), (48, 72, 12, 12, 160), (16, 64, 28, 28, 96),
+                  (8, 32, 33, 17, 1000)]
 
 
 @pytest.mark.parametrize("prec", ["f16", "bf16"])
@@ -562,11 +565,14 @@ def test_reduced_precision_assembly_kernels(ocn, oracle, torch_gpu, prec, N, C, 
         assert rel <= REL_L2_QUANTISED_RESTATEMENT, f"rel-L2 vs quantised restatement {rel:.3e}"
 
 
-def test_reduced_precision_assembly_variant_rejects_other_shapes(ocn, torch_gpu):
-    x, w = make_tensors(ocn, 32, 16, 6, 6, 96)  # K % 64 != 0: the HIP kernel's shape
+def test_reduced_precision_assembly_variant_needs_the_balanced_split(ocn, torch_gpu):
+    # 400 workgroup tiles on 256 compute units: the persistent launch cuts tiles, which the caller
+    # has switched off, so the assembly kernel selected explicitly must refuse (no silent fallback)
+    x, w = make_tensors(ocn, 32, 16, 40, 40, 128)
     r = Runner(ocn, torch_gpu, x, w)
     try:
         ocn.set_operand_precision(ocn.F16)
+        ocn.set_balanced_split(False)
         ocn.set_kernel_variant(ocn.KERNEL_ASM)
         with pytest.raises(ocn.OpenCNNError):
             r.dropin()
@@ -574,6 +580,7 @@ def test_reduced_precision_assembly_variant_rejects_other_shapes(ocn, torch_gpu)
         assert not np.isnan(r.dropin()).any()
     finally:
         ocn.set_kernel_variant(ocn.KERNEL_AUTO)
+        ocn.set_balanced_split(True)
         ocn.set_operand_precision(ocn.F32)
 
 
