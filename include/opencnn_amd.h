@@ -132,10 +132,11 @@ int opencnn_set_stream(void *stream);
  *                            filter groups, otherwise later launches return
  *                            hipErrorInvalidValue)
  *   OPENCNN_KERNEL_ASM       the LDS scheme as hand-scheduled gfx950 assembly, one persistent
- *                            launch over all (tile, 8-channel chunk) units.  Needs an even number
- *                            of 32-wide filter groups (and, for more workgroup tiles than compute
- *                            units that are not a multiple of them, the balanced split switched
- *                            on); otherwise later launches return hipErrorInvalidValue.
+ *                            launch over all (tile, 8-channel chunk) units.  Needs more than one
+ *                            32-wide filter group, i.e. filt_k > 32 (and, for more workgroup
+ *                            tiles than compute units that are not a multiple of them, the
+ *                            balanced split switched on); otherwise later launches return
+ *                            hipErrorInvalidValue.
  *                            With fp16 / bf16 operands (opencnn_set_operand_precision): units of
  *                            16 channels, any shape (the condition on the balanced split
  *                            stays)

@@ -487,28 +487,41 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
     return launch_h16(a, precision, st);
   }
 
-  // Waves per workgroup that share one column tile (and split its input transform): as many as
-  // the (rounded-up) filter groups fill whole workgroups of.
   const bool ragged = ragged_shape(in_n, in_c, filt_k);
   const int variant = g_variant.load();
+  // kw = waves per workgroup that share one column tile (and split its input transform); the
+  // workgroup's other dimension is 4 / kw column tiles.
+  auto tile_with = [&a](int kw) {
+    const int cw = 4 / kw;
+    const long long colblocks = (a.colgroups + cw - 1) / cw;
+    const long long nblocks = colblocks * ((a.kgroups + kw - 1) / kw);
+    if (nblocks > kMaxElems / 8) return false;
+    a.nblocks = (int)nblocks;
+    a.colblocks = (int)colblocks;
+    return true;
+  };
+  auto lds_bytes = [](int kw) { return (size_t)(4 / kw) * 2 * 4 * 16 * 64 * sizeof(float); };
+
+  if (variant == OPENCNN_KERNEL_ASM || variant == OPENCNN_KERNEL_AUTO) {
+    // The assembly kernels take a last filter block with fewer than kw filter groups: a wave
+    // without filters reads zeros past the end of Ww, multiplies them and stores no row (the
+    // row masks of the _ragged kernels).  So: the kw that leaves the fewest such waves, 4 on a tie.
+    // A single filter group would idle half of the matrix pipes: the register variant below
+    // is faster there (measured, K = 32).
+    const int kw = a.kgroups == 1 ? 1 : ((a.kgroups + 3) / 4 * 4 <= (a.kgroups + 1) / 2 * 2 ? 4 : 2);
+    REQUIRE(tile_with(kw));
+    int grid = 0;
+    if (int e = asm_grid(a, kw, (a.C + 7) / 8, &grid)) return e;
+    if (grid > 0) return launch_asm(a, kw, grid, ragged || a.kgroups % kw != 0, lds_bytes(kw), st);
+    REQUIRE(variant != OPENCNN_KERNEL_ASM);
+  }
+  // The HIP C++ kernels: as many sharing waves as the (rounded-up) filter groups fill whole
+  // workgroups of.
   int kw = 1;
   if (variant != OPENCNN_KERNEL_REGISTER) kw = a.kgroups % 4 == 0 ? 4 : (a.kgroups % 2 == 0 ? 2 : 1);
   if (variant == OPENCNN_KERNEL_LDS) REQUIRE(kw > 1);
-  const int cw = 4 / kw;
-  const long long colblocks = (a.colgroups + cw - 1) / cw;
-  const long long nblocks = colblocks * (a.kgroups / kw);
-  REQUIRE(nblocks <= kMaxElems / 8);
-  a.nblocks = (int)nblocks;
-  a.colblocks = (int)colblocks;
-  const size_t lds_bytes = (size_t)cw * 2 * 4 * 16 * 64 * sizeof(float);
-
-  if (variant == OPENCNN_KERNEL_ASM || variant == OPENCNN_KERNEL_AUTO) {
-    int grid = 0;
-    if (int e = asm_grid(a, kw, (a.C + 7) / 8, &grid)) return e;
-    if (grid > 0) return launch_asm(a, kw, grid, ragged, lds_bytes, st);
-    REQUIRE(variant != OPENCNN_KERNEL_ASM);
-  }
-  return launch_hip(a, kw, ragged, variant != OPENCNN_KERNEL_LDS, lds_bytes, st);
+  REQUIRE(tile_with(kw));
+  return launch_hip(a, kw, ragged, variant != OPENCNN_KERNEL_LDS, lds_bytes(kw), st);
 }
 
 }  // namespace

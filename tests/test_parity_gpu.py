@@ -318,7 +318,12 @@ def test_balanced_split_matches_plain_launch(ocn, oracle, torch_gpu, N, C, H, K,
 ASM_SHAPES = [(32, 8, 8, 8, 64), (64, 64, 8, 8, 64), (64, 16, 7, 15, 64), (32, 8, 7, 15, 256),
               (64, 32, 16, 16, 128), (64, 24, 31, 31, 64), (32, 40, 45, 45, 64), (32, 16, 63, 5, 128),
               (32, 8, 1, 1, 64), (32, 16, 3, 5, 128), (96, 40, 21, 27, 64), (32, 8, 112, 112, 64),
-              (32, 1024, 7, 7, 1024), (256, 64, 28, 28, 64)]
+              (32, 1024, 7, 7, 1024), (256, 64, 28, 28, 64),
+              # 3, 5, 7, 9 filter groups: the last filter block has waves without filters
+              (32, 8, 6, 6, 96), (64, 96, 28, 28, 96), (64, 40, 14, 14, 160), (64, 32, 20, 20, 224),
+              (32, 24, 30, 30, 288),
+              # the same with nothing dividing
+              (40, 20, 9, 9, 70), (33, 9, 11, 11, 130)]
 
 
 @pytest.mark.parametrize("N,C,H,W,K", ASM_SHAPES)
@@ -356,14 +361,19 @@ def test_benchmark_configs_on_hip_kernels(ocn, oracle, torch_gpu, name, N, C, H,
     check_against_oracle(oracle, y, x, w)
 
 
-def test_assembly_variant_rejects_shapes_it_does_not_take(ocn, torch_gpu):
-    x, w = make_tensors(ocn, 32, 8, 6, 6, 96)  # three filter groups: no whole filter block
+def test_assembly_variant_rejects_launches_it_does_not_take(ocn, torch_gpu):
+    # 450 workgroup tiles on 256 compute units need the balanced split, which is switched off
+    x, w = make_tensors(ocn, 32, 8, 60, 60, 64)
     r = Runner(ocn, torch_gpu, x, w)
     try:
         ocn.set_kernel_variant(ocn.KERNEL_ASM)
+        ocn.set_balanced_split(False)
         with pytest.raises(ocn.OpenCNNError):
             r.dropin()
+        ocn.set_kernel_variant(ocn.KERNEL_AUTO)
+        assert not np.isnan(r.dropin()).any()
     finally:
+        ocn.set_balanced_split(True)
         ocn.set_kernel_variant(ocn.KERNEL_AUTO)
 
 
