@@ -49,7 +49,7 @@ extern "C" const char opencnn_wino_h16_asm_hsaco[];  // gen_wino_h16_asm.py
 struct AsmKernels {
   hipModule_t module = nullptr, module_h16 = nullptr;
   hipFunction_t kw2 = nullptr, kw4 = nullptr, kw2_ragged = nullptr, kw4_ragged = nullptr;
-  hipFunction_t f16_kw4 = nullptr, bf16_kw4 = nullptr;
+  hipFunction_t f16_kw4 = nullptr, bf16_kw4 = nullptr, f16_kw4_ragged = nullptr, bf16_kw4_ragged = nullptr;
   unsigned* split_sync = nullptr;  // device address of g_split_sync (all sets) on this device
   bool ready = false;
 };
@@ -73,6 +73,8 @@ int asm_kernels(const AsmKernels** out) {
     if ((e = hipModuleLoadData(&k.module_h16, opencnn_wino_h16_asm_hsaco)) != hipSuccess) return (int)e;
     if ((e = hipModuleGetFunction(&k.f16_kw4, k.module_h16, "wino_f16_asm_kw4")) != hipSuccess) return (int)e;
     if ((e = hipModuleGetFunction(&k.bf16_kw4, k.module_h16, "wino_bf16_asm_kw4")) != hipSuccess) return (int)e;
+    if ((e = hipModuleGetFunction(&k.f16_kw4_ragged, k.module_h16, "wino_f16_asm_kw4_ragged")) != hipSuccess) return (int)e;
+    if ((e = hipModuleGetFunction(&k.bf16_kw4_ragged, k.module_h16, "wino_bf16_asm_kw4_ragged")) != hipSuccess) return (int)e;
     if ((e = hipGetSymbolAddress(reinterpret_cast<void**>(&k.split_sync), HIP_SYMBOL(opencnn::g_split_sync))) != hipSuccess)
       return (int)e;
     // 64 KB of dynamic LDS for KW = 2 is the default limit exactly; nothing to raise
@@ -363,9 +365,9 @@ constexpr int kEpilogueHalfUnits = 3;
 int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* launched) {
   *launched = false;
   // Any shape.  Waves of the last filter block whose 32 filters do not exist help with the input
-  // transform, multiply zeros and store nothing; the last chunk's missing channels read as zeros
-  // (descriptor cut at the tensor's end) and meet zero rows of the padded transformed filter;
-  // batch elements and filter rows that do not exist are masked per lane / per row.
+  // transform, multiply zeros and store nothing.  In the _ragged kernels the last chunk's missing
+  // channels read as zeros (descriptor cut at the tensor's end) and meet zero rows of the padded
+  // transformed filter; batch elements and filter rows that do not exist are masked per lane / row.
   if ((long long)a.N * a.H * a.W * 4 * 4 > kMaxElems) return 0;  // four-channel slab in bytes
   const int kblocks = (a.kgroups + 3) / 4, chunks = (int)(padded_c_h16(a.C) / 16);
   const long long nblocks = (long long)a.colgroups * kblocks;
@@ -380,7 +382,12 @@ int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* lau
   const AsmKernels* ak = nullptr;
   if (int e = asm_kernels(&ak)) return e;
   AsmLaunch l;
-  l.fn = precision == OPENCNN_BF16 ? ak->bf16_kw4 : ak->f16_kw4;
+  // the _ragged kernels mask batch elements, channels and filter rows that do not exist
+  const bool ragged = a.N % 32 != 0 || a.C % 16 != 0 || a.K % 32 != 0;
+  if (precision == OPENCNN_BF16)
+    l.fn = ragged ? ak->bf16_kw4_ragged : ak->bf16_kw4;
+  else
+    l.fn = ragged ? ak->f16_kw4_ragged : ak->f16_kw4;
   l.grid = grid;
   l.lds_bytes = 2 * 16 * 2 * 4 * 32 * sizeof(unsigned);  // two buffers of V
   l.chunks = chunks;

@@ -29,9 +29,10 @@ What differs from the fp32 kernels:
   * s_waitcnt counts are derived by the generator from the issue order of the loads.
 
 Any N, C, K (api.hip pads the transformed filter with zeros to whole chunks of 16 channels and
-pairs of 32-wide filter groups): batch elements and filter rows that do not exist are masked as
-in the _ragged fp32 kernels, the last chunk's slab ends with the tensor (slab_descriptor), waves
-of the last filter block without filters load and store nothing (filter_descriptor).
+pairs of 32-wide filter groups).  In every kernel, waves of the last filter block without filters
+load and store nothing (filter_descriptor); the _ragged kernels also mask batch elements and
+filter rows that do not exist, as the _ragged fp32 kernels do, and end the last chunk's slab with
+the tensor (slab_descriptor).
 
 Usage: gen_wino_h16_asm.py > wino_h16_asm.s
 """
@@ -54,13 +55,15 @@ class KernelH16(Kernel):
     SLAB_CHANNELS = 4
     K_REAL = "Q"  # the argument slot Q (twice the chunks per tile in the fp32 kernels) carries K here
 
-    def __init__(self, bf16):
+    def __init__(self, bf16, ragged=False):
+        """ragged: shapes outside N % 32 == 0, C % 16 == 0, K % 32 == 0 (masked lanes and rows, a
+        slab descriptor that ends with the tensor; a few scalar instructions per unit and row)."""
         self.bf16 = bf16
         self.KW, self.CW, self.SPW = 4, 1, 1
-        self.ragged = False
-        self.ragged_n = self.ragged_k = True  # any N, K: a handful of scalar instructions per tile
+        self.ragged = False  # the fp32 kernels' two-channel slab logic is replaced, see slab_descriptor
+        self.ragged_c = self.ragged_n = self.ragged_k = ragged
         self.lines, self.outofline, self.nlabel = [], [], 0
-        self.name = f"wino_{'bf16' if bf16 else 'f16'}_asm_kw4"
+        self.name = f"wino_{'bf16' if bf16 else 'f16'}_asm_kw4" + ("_ragged" if ragged else "")
         self.alloc()
 
     # ------------------------------------------------------------------ registers
@@ -238,12 +241,13 @@ class KernelH16(Kernel):
         rx = self.S["RsrcX"]
         self.e(f"s_lshl_b32 {t(0)}, {self.sr('Cp')}, 2")
         self.e(f"s_add_u32 {t(0)}, {t(0)}, {self.sr('KwSpw')}")
-        self.e(f"s_abs_i32 {t(2)}, {self.sr('Creal')}")
-        self.e(f"s_lshl_b32 {t(1)}, {t(0)}, 2")
-        self.e(f"s_sub_i32 {t(2)}, {t(2)}, {t(1)}")
-        self.e(f"s_max_i32 {t(2)}, {t(2)}, 0")
-        self.e(f"s_min_i32 {t(2)}, {t(2)}, 4")
-        self.e(f"s_mul_i32 {s(rx + 2)}, {t(2)}, {self.sr('HWN4')}")
+        if self.ragged_c:
+            self.e(f"s_abs_i32 {t(2)}, {self.sr('Creal')}")
+            self.e(f"s_lshl_b32 {t(1)}, {t(0)}, 2")
+            self.e(f"s_sub_i32 {t(2)}, {t(2)}, {t(1)}")
+            self.e(f"s_max_i32 {t(2)}, {t(2)}, 0")
+            self.e(f"s_min_i32 {t(2)}, {t(2)}, 4")
+            self.e(f"s_mul_i32 {s(rx + 2)}, {t(2)}, {self.sr('HWN4')}")
         self.e(f"s_mul_hi_u32 {t(1)}, {t(0)}, {self.sr('Slab')}")
         self.e(f"s_mul_i32 {t(0)}, {t(0)}, {self.sr('Slab')}")
         self.e(f"s_add_u32 {s(rx)}, {s(self.S['X'])}, {t(0)}")
@@ -618,7 +622,7 @@ class KernelH16(Kernel):
 
 def main():
     out = ['\t.amdgcn_target "amdgcn-amd-amdhsa--gfx950"', "\t.amdhsa_code_object_version 6"]
-    kernels = [KernelH16(False), KernelH16(True)]
+    kernels = [KernelH16(bf16, ragged) for ragged in (False, True) for bf16 in (False, True)]
     for k in kernels:
         k.emit(out)
     out.append("\t.amdgpu_metadata\n---\namdhsa.kernels:")

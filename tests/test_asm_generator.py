@@ -89,9 +89,10 @@ def gen_h16(gen):
     return mod
 
 
+@pytest.mark.parametrize("ragged", [False, True])
 @pytest.mark.parametrize("bf16", [False, True])
-def test_h16_register_budget(gen_h16, bf16):
-    k = gen_h16.KernelH16(bf16)
+def test_h16_register_budget(gen_h16, bf16, ragged):
+    k = gen_h16.KernelH16(bf16, ragged)
     assert k.vgpr_count <= 256
     assert k.sgpr_count <= 98
     assert len(set(k.MP)) == 64
@@ -104,11 +105,15 @@ def test_h16_register_budget(gen_h16, bf16):
     assert k.V["U"] % 2 == 0 and k.V["VR"] % 2 == 0
 
 
+@pytest.mark.parametrize("ragged", [False, True])
 @pytest.mark.parametrize("bf16", [False, True])
-def test_h16_kernel_text_invariants(gen_h16, bf16):
-    k = gen_h16.KernelH16(bf16)
+def test_h16_kernel_text_invariants(gen_h16, bf16, ragged):
+    k = gen_h16.KernelH16(bf16, ragged)
     k.body()
     text = "\n".join(k.lines)
+    assert k.name.endswith("_ragged") == ragged
+    # lane masks (batch elements that do not exist) only in the _ragged kernels
+    assert ("v_cndmask_b32" in text) == ragged
     op = "v_mfma_f32_32x32x16_bf16" if bf16 else "v_mfma_f32_32x32x16_f16"
     other = "v_mfma_f32_32x32x16_f16" if bf16 else "v_mfma_f32_32x32x16_bf16"
     # six chunk bodies (plain first / merging first / steady state, each for even and odd units)
