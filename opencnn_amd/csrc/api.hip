@@ -357,8 +357,9 @@ int launch_asm(const opencnn::ConvArgs& a, int kw, int grid, bool ragged, size_t
   return launch_asm_kernel(a, l, st);
 }
 
-// The hand-scheduled fp16 / bf16 kernels (gen_wino_h16_asm.py) take whole 128-filter blocks and
-// 16-channel chunks of shapes inside the reference's tiling; *launched stays false otherwise.
+// The hand-scheduled fp16 / bf16 kernels (gen_wino_h16_asm.py): 128-filter blocks, 16-channel
+// chunks.  *launched stays false when the launch does not fit them (sizes beyond 31-bit offsets,
+// a tile count that needs the balanced split while it is switched off).
 // An output transform of the fp16 / bf16 kernels takes about as long as 1.5 of their units.
 constexpr int kEpilogueHalfUnits = 3;
 
