@@ -2,7 +2,8 @@
  * opencnn_amd — C ABI of the MI355X (gfx950) Winograd F(2x2,3x3) forward convolution.
  *
  * Plain C: pointers and sizes only.  Every device pointer is memory the CALLER
- * allocated on the current HIP device; the library allocates no tensors or workspaces.  Its
+ * allocated on the current HIP device (any float-aligned address, e.g. a slice of a larger
+ * allocation); the library allocates no tensors or workspaces.  Its
  * state between calls is the process-wide settings of the opencnn_set_* calls below (stream,
  * kernel variant, balanced split, operand precision), the code objects of its assembly kernels
  * (embedded in the library, loaded once per device by opencnn_init or the first launch) and

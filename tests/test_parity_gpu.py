@@ -377,6 +377,39 @@ def test_assembly_variant_rejects_launches_it_does_not_take(ocn, torch_gpu):
         ocn.set_kernel_variant(ocn.KERNEL_AUTO)
 
 
+@pytest.mark.parametrize("family", ["auto", "hip"])
+@pytest.mark.parametrize("prec", ["f32", "f16"])
+@pytest.mark.parametrize("N,C,H,K", [(64, 64, 14, 64), (128, 64, 20, 128), (33, 20, 9, 100)])
+def test_buffers_need_only_float_alignment(ocn, oracle, torch_gpu, family, prec, N, C, H, K):
+    # sub-tensors of a larger allocation: every pointer 4, 8 or 12 bytes past a 16-byte boundary
+    # (the kernels' wide loads and stores must not assume more than the element's alignment)
+    torch = torch_gpu
+    x, w = make_tensors(ocn, N, C, H, H, K)
+    ref = oracle.direct_conv_f64(x, w)
+    n_out, n_ws = K * H * H * N, ocn.workspace_bytes(C, K) // 4
+    for off in (1, 2, 3):
+        print(f"alignment {family} {prec} N={N} C={C} H={H} K={K} offset {off}", flush=True)
+        xd = torch.zeros(x.size + 8, device="cuda")[off:off + x.size]
+        xd.copy_(torch.from_numpy(x.ravel()))
+        wd = torch.zeros(w.size + 8, device="cuda")[off:off + w.size]
+        wd.copy_(torch.from_numpy(w.ravel()))
+        raw = torch.full((n_out + 8,), float("nan"), device="cuda")
+        ws = torch.zeros(n_ws + 8, device="cuda")[off:off + n_ws]
+        try:
+            ocn.set_kernel_variant(ocn.KERNEL_AUTO if family == "auto" else ocn.KERNEL_HIP)
+            ocn.set_operand_precision(ocn.F32 if prec == "f32" else ocn.F16)
+            ocn.filter_transform(wd, ws, K, C, ocn.FILTER_CRSK, ocn.WW_MFMA)
+            ocn.conv_forward_pretransformed(xd, ws, raw[off:off + n_out], N, C, H, H, K)
+            torch.cuda.synchronize()
+        finally:
+            ocn.set_kernel_variant(ocn.KERNEL_AUTO)
+            ocn.set_operand_precision(ocn.F32)
+        r = raw.cpu().numpy()
+        assert np.isnan(r[:off]).all() and np.isnan(r[off + n_out:]).all(), "wrote outside the output"
+        rel, _, _ = oracle.compare(r[off:off + n_out].reshape(K, H, H, N), ref)
+        assert rel <= (1e-5 if prec == "f32" else 2e-3), f"rel-L2 vs fp64 direct {rel:.3e}"
+
+
 # ---------------------------------------------------------------- shapes outside the reference's tiling
 
 RAGGED = [
