@@ -133,7 +133,8 @@ int opencnn_set_stream(void *stream);
  *                            filter groups, otherwise later launches return
  *                            hipErrorInvalidValue)
  *   OPENCNN_KERNEL_ASM       the LDS scheme as hand-scheduled gfx950 assembly, one persistent
- *                            launch over all (tile, 8-channel chunk) units.  Needs more than one
+ *                            launch over all (tile, 8-channel chunk) units (batches of 16 and
+ *                            fewer: several spatial tiles share a 32-column tile).  Needs more than one
  *                            32-wide filter group, i.e. filt_k > 32 (and, for more workgroup
  *                            tiles than compute units that are not a multiple of them, the
  *                            balanced split switched on); otherwise later launches return

@@ -49,7 +49,9 @@ extern "C" const char opencnn_wino_h16_asm_hsaco[];  // gen_wino_h16_asm.py
 struct AsmKernels {
   hipModule_t module = nullptr, module_h16 = nullptr;
   hipFunction_t kw2 = nullptr, kw4 = nullptr, kw2_ragged = nullptr, kw4_ragged = nullptr;
+  hipFunction_t kw2_packed = nullptr, kw4_packed = nullptr;
   hipFunction_t f16_kw4 = nullptr, bf16_kw4 = nullptr, f16_kw4_ragged = nullptr, bf16_kw4_ragged = nullptr;
+  hipFunction_t f16_kw4_packed = nullptr, bf16_kw4_packed = nullptr;
   unsigned* split_sync = nullptr;  // device address of g_split_sync (all sets) on this device
   bool ready = false;
 };
@@ -70,11 +72,15 @@ int asm_kernels(const AsmKernels** out) {
     if ((e = hipModuleGetFunction(&k.kw4, k.module, "wino_f32_asm_kw4")) != hipSuccess) return (int)e;
     if ((e = hipModuleGetFunction(&k.kw2_ragged, k.module, "wino_f32_asm_kw2_ragged")) != hipSuccess) return (int)e;
     if ((e = hipModuleGetFunction(&k.kw4_ragged, k.module, "wino_f32_asm_kw4_ragged")) != hipSuccess) return (int)e;
+    if ((e = hipModuleGetFunction(&k.kw2_packed, k.module, "wino_f32_asm_kw2_packed")) != hipSuccess) return (int)e;
+    if ((e = hipModuleGetFunction(&k.kw4_packed, k.module, "wino_f32_asm_kw4_packed")) != hipSuccess) return (int)e;
     if ((e = hipModuleLoadData(&k.module_h16, opencnn_wino_h16_asm_hsaco)) != hipSuccess) return (int)e;
     if ((e = hipModuleGetFunction(&k.f16_kw4, k.module_h16, "wino_f16_asm_kw4")) != hipSuccess) return (int)e;
     if ((e = hipModuleGetFunction(&k.bf16_kw4, k.module_h16, "wino_bf16_asm_kw4")) != hipSuccess) return (int)e;
     if ((e = hipModuleGetFunction(&k.f16_kw4_ragged, k.module_h16, "wino_f16_asm_kw4_ragged")) != hipSuccess) return (int)e;
     if ((e = hipModuleGetFunction(&k.bf16_kw4_ragged, k.module_h16, "wino_bf16_asm_kw4_ragged")) != hipSuccess) return (int)e;
+    if ((e = hipModuleGetFunction(&k.f16_kw4_packed, k.module_h16, "wino_f16_asm_kw4_packed")) != hipSuccess) return (int)e;
+    if ((e = hipModuleGetFunction(&k.bf16_kw4_packed, k.module_h16, "wino_bf16_asm_kw4_packed")) != hipSuccess) return (int)e;
     if ((e = hipGetSymbolAddress(reinterpret_cast<void**>(&k.split_sync), HIP_SYMBOL(opencnn::g_split_sync))) != hipSuccess)
       return (int)e;
     // 64 KB of dynamic LDS for KW = 2 is the default limit exactly; nothing to raise
@@ -289,6 +295,9 @@ struct AsmLaunch {
   // fp16 / bf16 kernels (>= 0): cost of an output transform in half units; ranges are then cut on
   // a weighted line, a tile = 2 * chunks + this, and the kernel maps positions back to units.
   int filters = -1;  // fp16 / bf16 kernels: the real filter count
+  // _packed kernels (>= 0): log2 of the batch elements per column tile; a column tile then holds
+  // 32 >> packed_log2 consecutive spatial tiles (batches of 16 and fewer).
+  int packed_log2 = -1;
   int epilogue_half_units = -1;
 };
 
@@ -304,7 +313,7 @@ int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmLaunch& l, hipStream_
   ka.W = a.W;
   ka.chunks = chunks;
   ka.tiles_w = a.tiles_w;
-  ka.ngroups = a.ngroups;
+  ka.ngroups = l.packed_log2 >= 0 ? l.packed_log2 : a.ngroups;
   ka.colgroups = a.colgroups;
   ka.colblocks = l.tile_split;
   ka.Q = l.filters >= 0 ? l.filters : chunks * 2;
@@ -334,6 +343,7 @@ int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmLaunch& l, hipStream_
   magic_divisor((uint32_t)l.tile_split, &ka.m_colblocks, &ka.s_colblocks);
   if (l.lockstep_log2 >= 0) ka.s_colblocks = (uint32_t)l.lockstep_log2;
   magic_divisor((uint32_t)a.ngroups, &ka.m_ngroups, &ka.s_ngroups);
+  if (l.packed_log2 >= 0) ka.m_ngroups = (uint32_t)(a.tiles_h * a.tiles_w);  // the spatial tiles
   magic_divisor((uint32_t)a.tiles_w, &ka.m_tiles_w, &ka.s_tiles_w);
   size_t ka_size = sizeof(ka);
   void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &ka, HIP_LAUNCH_PARAM_BUFFER_SIZE, &ka_size,
@@ -342,12 +352,30 @@ int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmLaunch& l, hipStream_
                                     nullptr, extra);
 }
 
-int launch_asm(const opencnn::ConvArgs& a, int kw, int grid, bool ragged, size_t lds_bytes,
+// Batches of 16 and fewer: the assembly kernels fill the 32 columns of a column tile with
+// NB = 2^k >= N batch elements of 32 / NB consecutive spatial tiles (_packed kernels) instead of
+// leaving columns empty.  Returns log2 NB, or -1 for larger batches; *a gets the packed column
+// tiles.
+int pack_columns(opencnn::ConvArgs* a) {
+  if (a->N > 16) return -1;
+  int log2nb = 0;
+  while ((1 << log2nb) < a->N) ++log2nb;
+  const int per_tile = 32 >> log2nb;
+  a->ngroups = 1;
+  a->colgroups = (a->tiles_h * a->tiles_w + per_tile - 1) / per_tile;
+  return log2nb;
+}
+
+int launch_asm(const opencnn::ConvArgs& a, int kw, int grid, bool ragged, int packed_log2, size_t lds_bytes,
                hipStream_t st) {
   const AsmKernels* ak = nullptr;
   if (int e = asm_kernels(&ak)) return e;
   AsmLaunch l;
-  l.fn = ragged ? (kw == 4 ? ak->kw4_ragged : ak->kw2_ragged) : (kw == 4 ? ak->kw4 : ak->kw2);
+  if (packed_log2 >= 0)
+    l.fn = kw == 4 ? ak->kw4_packed : ak->kw2_packed;
+  else
+    l.fn = ragged ? (kw == 4 ? ak->kw4_ragged : ak->kw2_ragged) : (kw == 4 ? ak->kw4 : ak->kw2);
+  l.packed_log2 = packed_log2;
   l.grid = grid;
   l.lds_bytes = lds_bytes;
   l.chunks = (a.C + 7) / 8;
@@ -365,6 +393,7 @@ constexpr int kEpilogueHalfUnits = 3;
 
 int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* launched) {
   *launched = false;
+  const int packed_log2 = pack_columns(&a);
   // Any shape.  Waves of the last filter block whose 32 filters do not exist help with the input
   // transform, multiply zeros and store nothing.  In the _ragged kernels the last chunk's missing
   // channels read as zeros (descriptor cut at the tensor's end) and meet zero rows of the padded
@@ -386,9 +415,10 @@ int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* lau
   // the _ragged kernels mask batch elements, channels and filter rows that do not exist
   const bool ragged = a.N % 32 != 0 || a.C % 16 != 0 || a.K % 32 != 0;
   if (precision == OPENCNN_BF16)
-    l.fn = ragged ? ak->bf16_kw4_ragged : ak->bf16_kw4;
+    l.fn = packed_log2 >= 0 ? ak->bf16_kw4_packed : (ragged ? ak->bf16_kw4_ragged : ak->bf16_kw4);
   else
-    l.fn = ragged ? ak->f16_kw4_ragged : ak->f16_kw4;
+    l.fn = packed_log2 >= 0 ? ak->f16_kw4_packed : (ragged ? ak->f16_kw4_ragged : ak->f16_kw4);
+  l.packed_log2 = packed_log2;
   l.grid = grid;
   l.lds_bytes = 2 * 16 * 2 * 4 * 32 * sizeof(unsigned);  // two buffers of V
   l.chunks = chunks;
@@ -499,7 +529,7 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   const int variant = g_variant.load();
   // kw = waves per workgroup that share one column tile (and split its input transform); the
   // workgroup's other dimension is 4 / kw column tiles.
-  auto tile_with = [&a](int kw) {
+  auto tile_with = [](opencnn::ConvArgs& a, int kw) {
     const int cw = 4 / kw;
     const long long colblocks = (a.colgroups + cw - 1) / cw;
     const long long nblocks = colblocks * ((a.kgroups + kw - 1) / kw);
@@ -517,10 +547,13 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
     // A single filter group would idle half of the matrix pipes: the register variant below
     // is faster there (measured, K = 32).
     const int kw = a.kgroups == 1 ? 1 : ((a.kgroups + 3) / 4 * 4 <= (a.kgroups + 1) / 2 * 2 ? 4 : 2);
-    REQUIRE(tile_with(kw));
+    opencnn::ConvArgs b = a;
+    const int packed_log2 = pack_columns(&b);
+    REQUIRE(tile_with(b, kw));
     int grid = 0;
-    if (int e = asm_grid(a, kw, (a.C + 7) / 8, &grid)) return e;
-    if (grid > 0) return launch_asm(a, kw, grid, ragged || a.kgroups % kw != 0, lds_bytes(kw), st);
+    if (int e = asm_grid(b, kw, (b.C + 7) / 8, &grid)) return e;
+    if (grid > 0)
+      return launch_asm(b, kw, grid, ragged || b.kgroups % kw != 0, packed_log2, lds_bytes(kw), st);
     REQUIRE(variant != OPENCNN_KERNEL_ASM);
   }
   // The HIP C++ kernels: as many sharing waves as the (rounded-up) filter groups fill whole
@@ -528,7 +561,7 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   int kw = 1;
   if (variant != OPENCNN_KERNEL_REGISTER) kw = a.kgroups % 4 == 0 ? 4 : (a.kgroups % 2 == 0 ? 2 : 1);
   if (variant == OPENCNN_KERNEL_LDS) REQUIRE(kw > 1);
-  REQUIRE(tile_with(kw));
+  REQUIRE(tile_with(a, kw));
   return launch_hip(a, kw, ragged, variant != OPENCNN_KERNEL_LDS, lds_bytes(kw), st);
 }
 

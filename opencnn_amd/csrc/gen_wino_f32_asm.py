@@ -87,7 +87,7 @@ def a(i, n=1):
 class Kernel:
     K_REAL = "Kreal"  # the scalar register with the real filter count (ragged K)
 
-    def __init__(self, KW, ragged=False):
+    def __init__(self, KW, ragged=False, packed=False):
         """ragged: shapes outside N % 32 == 0, K % 32 == 0, C % 8 == 0.  Groups and chunks are
         rounded up by the host; lanes whose batch element does not exist read zeros and store
         nothing (out-of-range offsets), the last channel slab ends with the tensor, filter rows
@@ -96,12 +96,15 @@ class Kernel:
         self.ragged = ragged
         # batch elements, and filters, that do not exist are masked (the fp16 / bf16 kernels always do)
         self.ragged_n = self.ragged_k = ragged
+        # packed (batches of 16 and fewer, a _ragged kernel): the 32 columns of a column tile are
+        # NB = 2^k >= N batch elements of 32 / NB consecutive spatial tiles; see lane_tile
+        self.packed = packed
         self.CW = 4 // KW
         self.SPW = 4 // KW
         self.lines = []
         self.outofline = []  # rarely executed blocks, emitted behind s_endpgm
         self.nlabel = 0
-        self.name = f"wino_f32_asm_kw{KW}" + ("_ragged" if ragged else "")
+        self.name = f"wino_f32_asm_kw{KW}" + ("_packed" if packed else "_ragged" if ragged else "")
         self.alloc()
 
     # ------------------------------------------------------------------ helpers
@@ -201,6 +204,11 @@ class Kernel:
         self.e(f"s_cmp_lt_u32 {t(0)}, {self.sr('Colgroups')}")
         self.e(f"s_cselect_b32 {self.sr('Dlive')}, 1, 0")
         self.e(f"s_cselect_b32 {t(0)}, {t(0)}, {t(1)}")  # a missing column tile works on the last real one
+        if self.packed:  # the column tile is a group of spatial tiles; the lanes find their own
+            self.e(f"s_mov_b32 {self.sr('Dty')}, {t(0)}")
+            self.e(f"s_mov_b32 {self.sr('Dng')}, 0")
+            self.e(f"s_mov_b32 {self.sr('Dtx')}, 0")
+            return
         self.div(t(2), t(0), self.sr("Mng"), self.sr("Sng"))  # spatial tile
         self.e(f"s_mul_i32 {t(3)}, {t(2)}, {self.sr('Ngroups')}")
         self.e(f"s_sub_u32 {self.sr('Dng')}, {t(0)}, {t(3)}")
@@ -212,6 +220,8 @@ class Kernel:
         """Per-lane byte offsets of the 16 patch elements of the tile in D* (P cursor), relative to
         a two-channel slab; elements in the zero padding get an offset no num_records reaches."""
         t = self.t
+        if self.packed:
+            return self.patch_offsets_packed()
         self.e(f"s_lshl_b32 {t(0)}, {self.sr('Dty')}, 1")
         self.e(f"s_sub_i32 {t(0)}, {t(0)}, 1")  # first patch row
         self.e(f"s_lshl_b32 {t(1)}, {self.sr('Dtx')}, 1")
@@ -241,6 +251,104 @@ class Kernel:
                     self.e(f"s_add_i32 {t(3)}, {t(3)}, {self.sr('ColStep')}")
             if i < 3:
                 self.e(f"s_add_i32 {t(2)}, {t(2)}, {self.sr('RowStep')}")
+
+    # ------------------------------------------------------------------ packed column tiles (N <= 16)
+    # Column n32 of column tile g: batch element n32 & (NB - 1) of spatial tile g * (32 / NB) +
+    # (n32 >> log2 NB), tiles numbered row-major.  The argument slot Ngroups carries log2 NB, the
+    # slot Mng the number of spatial tiles.  Everything per lane happens here, at a tile switch:
+    # the units only see 16 patch offsets and 4 store offsets per lane, as before.  Scratch: the
+    # transform temporaries T, dead between two units.
+    def lane_tile(self):
+        """T[0] = batch element, T[1] = 2*ty, T[2] = 2*tx of this lane's tile in column tile Dty;
+        T[3] = 0, or the out-of-range bit for a lane whose tile or batch element does not exist."""
+        t = self.t
+        T = lambda i: self.vr("T", i)
+        self.e(f"v_and_b32 {T(0)}, 31, {self.vr('Lane')}")
+        self.e(f"v_lshrrev_b32 {T(1)}, {self.sr('Ngroups')}, {T(0)}")       # tile within the group
+        self.e(f"s_lshl_b32 {t(4)}, 1, {self.sr('Ngroups')}")
+        self.e(f"s_sub_u32 {t(4)}, {t(4)}, 1")
+        self.e(f"v_and_b32 {T(0)}, {t(4)}, {T(0)}")                         # batch element
+        self.e(f"s_lshr_b32 {t(4)}, 32, {self.sr('Ngroups')}")
+        self.e(f"s_mul_i32 {t(4)}, {t(4)}, {self.sr('Dty')}")
+        self.e(f"v_add_u32 {T(1)}, {t(4)}, {T(1)}")                         # spatial tile
+        self.e(f"v_cmp_gt_u32 vcc, {self.sr('Mng')}, {T(1)}")               # it exists
+        self.e(f"v_cndmask_b32 {T(3)}, {self.vr('Oob')}, {self.vr('Zero')}, vcc")
+        self.e(f"v_cmp_le_u32 vcc, {self.sr('N')}, {T(0)}")                 # the batch element does not
+        self.e(f"v_cndmask_b32 {T(3)}, {T(3)}, {self.vr('Oob')}, vcc")
+        # ty = tile / TilesW with the magic number, in 64 bits as the scalar div does
+        self.e(f"v_mul_lo_u32 {T(4)}, {T(1)}, {self.sr('Mtw')}")
+        self.e(f"v_mul_hi_u32 {T(5)}, {T(1)}, {self.sr('Mtw')}")
+        self.e(f"v_lshrrev_b64 {self.vr('T', 4, 2)}, {self.sr('Stw')}, {self.vr('T', 4, 2)}")
+        self.e(f"v_mul_lo_u32 {T(5)}, {T(4)}, {self.sr('TilesW')}")
+        self.e(f"v_sub_u32 {T(2)}, {T(1)}, {T(5)}")
+        self.e(f"v_lshlrev_b32 {T(1)}, 1, {T(4)}")
+        self.e(f"v_lshlrev_b32 {T(2)}, 1, {T(2)}")
+        self.e(f"v_lshlrev_b32 {T(0)}, 2, {T(0)}")                          # as a byte offset
+
+    def in_range(self, dst, x, limit, extra):
+        """dst = extra, or the out-of-range bit unless 0 <= x < limit (x a VGPR, limit an SGPR)."""
+        self.e(f"v_cmp_gt_u32 vcc, {limit}, {x}")  # unsigned: also rejects -1
+        self.e(f"v_cndmask_b32 {dst}, {self.vr('Oob')}, {extra}, vcc")
+
+    def patch_offsets_packed(self):
+        T = lambda i: self.vr("T", i)
+        self.lane_tile()
+        # T[4..7]: the four patch rows' bad bits (with the lane's), T[8..11]: the columns'
+        for i in range(4):
+            self.e(f"v_add_u32 {T(12)}, {i - 1}, {T(1)}")
+            self.in_range(T(4 + i), T(12), self.sr("H"), T(3))
+        for j in range(4):
+            self.e(f"v_add_u32 {T(12)}, {j - 1}, {T(2)}")
+            self.in_range(T(8 + j), T(12), self.sr("W"), self.vr("Zero"))
+        # element (0, 0): ((2ty - 1) * W + 2tx - 1) * N * 4 + n * 4 + the lane's channel
+        self.e(f"v_and_b32 {T(12)}, 31, {self.vr('Lane')}")
+        self.e(f"v_lshlrev_b32 {T(12)}, 2, {T(12)}")
+        self.e(f"v_sub_u32 {T(12)}, {self.vr('LaneX')}, {T(12)}")           # the channel part of LaneX
+        self.e(f"v_add_u32 {T(12)}, {T(12)}, {T(0)}")
+        self.e(f"v_add_u32 {T(13)}, -1, {T(1)}")
+        self.e(f"v_mul_lo_u32 {T(13)}, {T(13)}, {self.sr('RowStep')}")
+        self.e(f"v_add_u32 {T(12)}, {T(12)}, {T(13)}")
+        self.e(f"v_add_u32 {T(13)}, -1, {T(2)}")
+        self.e(f"v_mul_lo_u32 {T(13)}, {T(13)}, {self.sr('ColStep')}")
+        self.e(f"v_add_u32 {T(12)}, {T(12)}, {T(13)}")
+        for i in range(4):
+            self.e(f"v_mov_b32 {T(13)}, {T(12)}")
+            for j in range(4):
+                self.e(f"v_or3_b32 {self.vr('VOFF', i * 4 + j)}, {T(13)}, {T(4 + i)}, {T(8 + j)}")
+                if j < 3:
+                    self.e(f"v_add_u32 {T(13)}, {self.sr('ColStep')}, {T(13)}")
+            if i < 3:
+                self.e(f"v_add_u32 {T(12)}, {self.sr('RowStep')}, {T(12)}")
+
+    def store_offsets_packed(self):
+        """Eff[0..3] of the M tile: the lane's four outputs relative to its filter row."""
+        t = self.t
+        T = lambda i: self.vr("T", i)
+        self.lane_tile()
+        self.e(f"s_cmp_lg_u32 {self.sr('Dlive')}, 0")
+        self.e(f"s_cselect_b32 {t(3)}, 0, 0x{OOB:x}")
+        self.e(f"v_or_b32 {T(3)}, {t(3)}, {T(3)}")
+        for d in range(2):
+            self.e(f"v_add_u32 {T(12)}, {d}, {T(1)}")
+            self.in_range(T(4 + d), T(12), self.sr("H"), T(3))
+            self.e(f"v_add_u32 {T(12)}, {d}, {T(2)}")
+            self.in_range(T(8 + d), T(12), self.sr("W"), self.vr("Zero"))
+        # output (0, 0): (2ty * W + 2tx) * N * 4 + n * 4 + the lane's filter-row part of Off[0]
+        self.e(f"v_and_b32 {T(12)}, 31, {self.vr('Lane')}")
+        self.e(f"v_lshlrev_b32 {T(12)}, 2, {T(12)}")
+        self.e(f"v_sub_u32 {T(12)}, {self.vr('Off', 0)}, {T(12)}")
+        self.e(f"v_add_u32 {T(12)}, {T(12)}, {T(0)}")
+        self.e(f"v_mul_lo_u32 {T(13)}, {T(1)}, {self.sr('RowStep')}")
+        self.e(f"v_add_u32 {T(12)}, {T(12)}, {T(13)}")
+        self.e(f"v_mul_lo_u32 {T(13)}, {T(2)}, {self.sr('ColStep')}")
+        self.e(f"v_add_u32 {T(12)}, {T(12)}, {T(13)}")
+        self.e(f"v_add_u32 {T(13)}, {self.sr('RowStep')}, {T(12)}")
+        self.e(f"v_or3_b32 {self.vr('Eff', 0)}, {T(12)}, {T(4)}, {T(8)}")
+        self.e(f"v_or3_b32 {self.vr('Eff', 2)}, {T(13)}, {T(5)}, {T(8)}")
+        self.e(f"v_add_u32 {T(12)}, {self.sr('ColStep')}, {T(12)}")
+        self.e(f"v_add_u32 {T(13)}, {self.sr('ColStep')}, {T(13)}")
+        self.e(f"v_or3_b32 {self.vr('Eff', 1)}, {T(12)}, {T(4)}, {T(9)}")
+        self.e(f"v_or3_b32 {self.vr('Eff', 3)}, {T(13)}, {T(5)}, {T(9)}")
 
     def alive_lanes(self):
         """vcc = lanes whose batch element Dng*32 + lane%32 exists (ragged N)."""
@@ -284,6 +392,15 @@ class Kernel:
         t = self.t
         self.e(f"s_lshl_b32 {t(0)}, {self.sr('Dkb')}, {self.KW.bit_length() - 1}")
         self.e(f"s_add_u32 {self.sr('KgM')}, {t(0)}, {self.sr('Kw')}")
+        yt = self.S["Yt"]
+        if self.packed:
+            self.store_offsets_packed()
+            self.e(f"s_lshl_b32 {t(0)}, {self.sr('KgM')}, 5")
+            self.e(f"s_mul_hi_u32 {t(1)}, {t(0)}, {self.sr('HWN4')}")
+            self.e(f"s_mul_i32 {t(0)}, {t(0)}, {self.sr('HWN4')}")
+            self.e(f"s_add_u32 {s(yt)}, {s(self.S['Y'])}, {t(0)}")
+            self.e(f"s_addc_u32 {s(yt + 1)}, {s(self.S['Y'] + 1)}, {t(1)}")
+            return
         # validity of the four outputs (odd H / W: the last tile row / column keeps one)
         self.e(f"s_lshl_b32 {t(0)}, {self.sr('Dty')}, 1")
         self.e(f"s_add_u32 {t(0)}, {t(0)}, 1")
@@ -303,7 +420,6 @@ class Kernel:
             if self.ragged_n:
                 self.e(f"v_cndmask_b32 {self.vr('Eff', q)}, {self.vr('Oob')}, {self.vr('Eff', q)}, vcc")
         # first row of the tile: y + kg*32*HWN4 + ((2ty*W + 2tx)*N + ng*32)*4
-        yt = self.S["Yt"]
         self.e(f"s_lshl_b32 {t(0)}, {self.sr('KgM')}, 5")
         self.e(f"s_mul_hi_u32 {t(1)}, {t(0)}, {self.sr('HWN4')}")
         self.e(f"s_mul_i32 {t(0)}, {t(0)}, {self.sr('HWN4')}")
@@ -922,7 +1038,8 @@ class Kernel:
 
 def main():
     out = ['\t.amdgcn_target "amdgcn-amd-amdhsa--gfx950"', "\t.amdhsa_code_object_version 6"]
-    kernels = [Kernel(2), Kernel(4), Kernel(2, ragged=True), Kernel(4, ragged=True)]
+    kernels = [Kernel(2), Kernel(4), Kernel(2, ragged=True), Kernel(4, ragged=True),
+               Kernel(2, ragged=True, packed=True), Kernel(4, ragged=True, packed=True)]
     for k in kernels:
         k.emit(out)
     out.append("\t.amdgpu_metadata\n---\namdhsa.kernels:")

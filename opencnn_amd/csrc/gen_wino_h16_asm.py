@@ -55,15 +55,18 @@ class KernelH16(Kernel):
     SLAB_CHANNELS = 4
     K_REAL = "Q"  # the argument slot Q (twice the chunks per tile in the fp32 kernels) carries K here
 
-    def __init__(self, bf16, ragged=False):
+    def __init__(self, bf16, ragged=False, packed=False):
         """ragged: shapes outside N % 32 == 0, C % 16 == 0, K % 32 == 0 (masked lanes and rows, a
-        slab descriptor that ends with the tensor; a few scalar instructions per unit and row)."""
+        slab descriptor that ends with the tensor; a few scalar instructions per unit and row).
+        packed: a _ragged kernel for batches of 16 and fewer (Kernel.lane_tile)."""
         self.bf16 = bf16
         self.KW, self.CW, self.SPW = 4, 1, 1
         self.ragged = False  # the fp32 kernels' two-channel slab logic is replaced, see slab_descriptor
         self.ragged_c = self.ragged_n = self.ragged_k = ragged
+        self.packed = packed
         self.lines, self.outofline, self.nlabel = [], [], 0
-        self.name = f"wino_{'bf16' if bf16 else 'f16'}_asm_kw4" + ("_ragged" if ragged else "")
+        self.name = (f"wino_{'bf16' if bf16 else 'f16'}_asm_kw4" +
+                     ("_packed" if packed else "_ragged" if ragged else ""))
         self.alloc()
 
     # ------------------------------------------------------------------ registers
@@ -622,7 +625,8 @@ class KernelH16(Kernel):
 
 def main():
     out = ['\t.amdgcn_target "amdgcn-amd-amdhsa--gfx950"', "\t.amdhsa_code_object_version 6"]
-    kernels = [KernelH16(bf16, ragged) for ragged in (False, True) for bf16 in (False, True)]
+    kernels = [KernelH16(bf16, ragged, packed) for ragged, packed in ((False, False), (True, False), (True, True))
+               for bf16 in (False, True)]
     for k in kernels:
         k.emit(out)
     out.append("\t.amdgpu_metadata\n---\namdhsa.kernels:")

@@ -22,9 +22,13 @@ def gen():
     return mod
 
 
+VARIANTS = [(False, False), (True, False), (True, True)]  # (ragged, packed)
+
+
+@pytest.mark.parametrize("ragged,packed", VARIANTS)
 @pytest.mark.parametrize("kw", [2, 4])
-def test_register_budget(gen, kw):
-    k = gen.Kernel(kw)
+def test_register_budget(gen, kw, ragged, packed):
+    k = gen.Kernel(kw, ragged, packed)
     assert k.vgpr_count <= 256          # arch VGPRs; the 256 accumulators are AGPRs
     assert k.sgpr_count <= 96           # + VCC and the reserved registers of the target = 102
     assert len(set(k.MP)) == 64         # landing registers of a published partial tile
@@ -36,11 +40,15 @@ def test_register_budget(gen, kw):
     assert not live_at_boundary & set(k.MP), "partial tile would land on live pipeline registers"
 
 
+@pytest.mark.parametrize("ragged,packed", VARIANTS)
 @pytest.mark.parametrize("kw", [2, 4])
-def test_kernel_text_invariants(gen, kw):
-    k = gen.Kernel(kw)
+def test_kernel_text_invariants(gen, kw, ragged, packed):
+    k = gen.Kernel(kw, ragged, packed)
     k.body()
     text = "\n".join(k.lines)
+    assert k.name.endswith("_packed" if packed else "_ragged" if ragged else f"kw{kw}")
+    # per-lane tiles (a 64-bit shift for the division by the tiles per row) only when packed
+    assert ("v_lshrrev_b64" in text) == packed
     # one workgroup barrier per chunk variant + the prologue; three chunk variants
     assert text.count("s_barrier") == 4
     # 64 MFMAs per chunk variant, plus the second copy of step 0 (MFMAs 1..15) that carries the
@@ -89,10 +97,10 @@ def gen_h16(gen):
     return mod
 
 
-@pytest.mark.parametrize("ragged", [False, True])
+@pytest.mark.parametrize("ragged,packed", VARIANTS)
 @pytest.mark.parametrize("bf16", [False, True])
-def test_h16_register_budget(gen_h16, bf16, ragged):
-    k = gen_h16.KernelH16(bf16, ragged)
+def test_h16_register_budget(gen_h16, bf16, ragged, packed):
+    k = gen_h16.KernelH16(bf16, ragged, packed)
     assert k.vgpr_count <= 256
     assert k.sgpr_count <= 98
     assert len(set(k.MP)) == 64
@@ -105,13 +113,14 @@ def test_h16_register_budget(gen_h16, bf16, ragged):
     assert k.V["U"] % 2 == 0 and k.V["VR"] % 2 == 0
 
 
-@pytest.mark.parametrize("ragged", [False, True])
+@pytest.mark.parametrize("ragged,packed", VARIANTS)
 @pytest.mark.parametrize("bf16", [False, True])
-def test_h16_kernel_text_invariants(gen_h16, bf16, ragged):
-    k = gen_h16.KernelH16(bf16, ragged)
+def test_h16_kernel_text_invariants(gen_h16, bf16, ragged, packed):
+    k = gen_h16.KernelH16(bf16, ragged, packed)
     k.body()
     text = "\n".join(k.lines)
-    assert k.name.endswith("_ragged") == ragged
+    assert k.name.endswith("_packed" if packed else "_ragged" if ragged else "kw4")
+    assert ("v_lshrrev_b64" in text) == packed
     # lane masks (batch elements that do not exist) only in the _ragged kernels
     assert ("v_cndmask_b32" in text) == ragged
     op = "v_mfma_f32_32x32x16_bf16" if bf16 else "v_mfma_f32_32x32x16_f16"

@@ -410,6 +410,40 @@ def test_buffers_need_only_float_alignment(ocn, oracle, torch_gpu, family, prec,
         assert rel <= (1e-5 if prec == "f32" else 2e-3), f"rel-L2 vs fp64 direct {rel:.3e}"
 
 
+# batches of 16 and fewer: the assembly kernels pack several spatial tiles into a column tile
+PACKED_SHAPES = [(1, 64, 14, 14, 64), (2, 16, 7, 9, 128), (3, 8, 5, 5, 64), (4, 32, 28, 28, 96),
+                 (5, 24, 13, 17, 100), (8, 256, 14, 14, 256), (9, 40, 6, 6, 250), (16, 64, 56, 56, 64),
+                 (16, 8, 1, 1, 64), (7, 3, 33, 20, 40), (1, 16, 112, 112, 64), (12, 20, 2, 3, 160)]
+
+
+@pytest.mark.parametrize("prec", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("N,C,H,W,K", PACKED_SHAPES)
+def test_small_batches_on_packed_column_tiles(ocn, oracle, torch_gpu, prec, N, C, H, W, K):
+    # the assembly kernels selected explicitly; against the fp64 direct convolution, the HIP C++
+    # kernels (which leave the columns of missing batch elements empty) and a second call
+    print(f"packed {prec} N={N} C={C} H={H} W={W} K={K}", flush=True)
+    x, w = make_tensors(ocn, N, C, H, W, K)
+    r = Runner(ocn, torch_gpu, x, w)
+    try:
+        ocn.set_operand_precision({"f32": ocn.F32, "f16": ocn.F16, "bf16": ocn.BF16}[prec])
+        ocn.set_kernel_variant(ocn.KERNEL_ASM)
+        y = r.split()
+        y2 = r.split()
+        ocn.set_kernel_variant(ocn.KERNEL_HIP)
+        y_hip = r.split()
+    finally:
+        ocn.set_kernel_variant(ocn.KERNEL_AUTO)
+        ocn.set_operand_precision(ocn.F32)
+    assert not np.isnan(y).any(), "an output element was never written"
+    assert np.array_equal(y, y2)
+    bound = {"f32": 1e-5, "f16": 2e-3, "bf16": 1.5e-2}[prec]
+    rel64, _, _ = oracle.compare(y, oracle.direct_conv_f64(x, w))
+    assert rel64 <= bound, f"rel-L2 vs fp64 direct {rel64:.3e}"
+    # same products, same fp32 sums per output (the split between workgroups may differ)
+    rel_hip, _, _ = oracle.compare(y, y_hip)
+    assert rel_hip <= 1e-6, f"rel-L2 vs the HIP kernel {rel_hip:.3e}"
+
+
 # ---------------------------------------------------------------- shapes outside the reference's tiling
 
 RAGGED = [
