@@ -133,8 +133,8 @@ int opencnn_set_stream(void *stream);
  *                            filter groups, otherwise later launches return
  *                            hipErrorInvalidValue)
  *   OPENCNN_KERNEL_ASM       the LDS scheme as hand-scheduled gfx950 assembly, one persistent
- *                            launch over all (tile, 8-channel chunk) units (batches of 16 and
- *                            fewer: several spatial tiles share a 32-column tile).  Needs more than one
+ *                            launch over all (tile, 8-channel chunk) units (batches that are no
+ *                            multiple of 32 may share 32-column tiles across spatial tiles).  Needs more than one
  *                            32-wide filter group, i.e. filt_k > 32 (and, for more workgroup
  *                            tiles than compute units that are not a multiple of them, the
  *                            balanced split switched on); otherwise later launches return
@@ -245,6 +245,15 @@ int opencnn_synth_filter(float *dst, int k, int c, int layout, unsigned long lon
 
 /* Name of the last failing check in this thread ("" if none): a short static string. */
 const char *opencnn_last_error(void);
+
+/*
+ * Name of the fused kernel that this thread's last successful launch used ("" before the first):
+ * a short static string such as "wino_f32_asm_kw2" or "wino_f16_asm_kw4_packed" (the assembly
+ * kernels' symbol names) or "wino_f32_fused_lds" (a HIP C++ kernel).  For logs and tests: which
+ * kernel family a shape ends up in is the library's choice (see opencnn_set_kernel_variant).
+ * No counterpart in the reference, whose single kernel is fixed at compile time.
+ */
+const char *opencnn_last_kernel(void);
 
 #ifdef __cplusplus
 }

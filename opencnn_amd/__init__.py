@@ -35,6 +35,7 @@ from .binding import (  # noqa: F401
     KERNEL_HIP,
     synth_filter,
     synth_input,
+    last_kernel,
     tiles_dim,
     time_forward,
     workspace_bytes,
@@ -57,6 +58,7 @@ __all__ = [
     "conv_forward_pretransformed",
     "filter_transform",
     "init",
+    "last_kernel",
     "lib",
     "load_library",
     "set_stream",

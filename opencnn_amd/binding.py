@@ -69,6 +69,7 @@ EXPORTED_SYMBOLS = {
          ctypes.c_double],
     ),
     "opencnn_last_error": (ctypes.c_char_p, []),
+    "opencnn_last_kernel": (ctypes.c_char_p, []),
 }
 
 
@@ -150,6 +151,11 @@ def _check(func: str, status: int) -> None:
 
 def init() -> None:
     _check("opencnn_init", lib().opencnn_init())
+
+
+def last_kernel() -> str:
+    """Name of the fused kernel this thread's last successful launch used."""
+    return lib().opencnn_last_kernel().decode()
 
 
 def tiles_dim(in_w: int) -> int:

@@ -41,6 +41,7 @@ int compute_units(int* out) {
   return 0;
 }
 thread_local const char* t_last_error = "";
+thread_local const char* t_last_kernel = "";
 
 // ---- hand-scheduled assembly kernels (gen_wino_f32_asm.py), loaded from the embedded code object
 extern "C" const char opencnn_wino_f32_asm_hsaco[];
@@ -135,6 +136,13 @@ void magic_divisor(uint32_t d, uint32_t* m, uint32_t* s) {
   while ((1ull << l) < d) ++l;
   *m = (uint32_t)(((1ull << (31 + l)) + d - 1) / d);
   *s = 31 + l;
+}
+
+// Result of a HIP C++ kernel launch; remembers the kernel's name on success.
+int launched_hip(const char* name) {
+  const hipError_t e = hipGetLastError();
+  if (e == hipSuccess) t_last_kernel = name;
+  return (int)e;
 }
 
 int fail(const char* what) {
@@ -257,7 +265,7 @@ int launch_h16(opencnn::ConvArgs a, int precision, hipStream_t st) {
     if (e != hipSuccess) return (int)e;
   }
   fn<<<grid, block, lds, st>>>(a);
-  return (int)hipGetLastError();
+  return launched_hip("wino_h16_fused_lds");
 }
 
 // Grid of the hand-scheduled kernels for this layer, or 0 when they do not take it.  One
@@ -281,6 +289,7 @@ int asm_grid(const opencnn::ConvArgs& a, int kw, int chunks, int* grid) {
 // One launch of a hand-scheduled kernel.
 struct AsmLaunch {
   hipFunction_t fn = nullptr;
+  const char* name = "";
   int grid = 0;
   size_t lds_bytes = 0;
   int chunks = 0;           // units per workgroup tile
@@ -295,9 +304,9 @@ struct AsmLaunch {
   // fp16 / bf16 kernels (>= 0): cost of an output transform in half units; ranges are then cut on
   // a weighted line, a tile = 2 * chunks + this, and the kernel maps positions back to units.
   int filters = -1;  // fp16 / bf16 kernels: the real filter count
-  // _packed kernels (>= 0): log2 of the batch elements per column tile; a column tile then holds
-  // 32 >> packed_log2 consecutive spatial tiles (batches of 16 and fewer).
-  int packed_log2 = -1;
+  // _packed kernels: the column tiles are cut from the line of all (spatial tile, batch element)
+  // pairs; the magic number of the image groups then divides by the batch size.
+  bool packed = false;
   int epilogue_half_units = -1;
 };
 
@@ -313,7 +322,7 @@ int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmLaunch& l, hipStream_
   ka.W = a.W;
   ka.chunks = chunks;
   ka.tiles_w = a.tiles_w;
-  ka.ngroups = l.packed_log2 >= 0 ? l.packed_log2 : a.ngroups;
+  ka.ngroups = a.ngroups;
   ka.colgroups = a.colgroups;
   ka.colblocks = l.tile_split;
   ka.Q = l.filters >= 0 ? l.filters : chunks * 2;
@@ -342,40 +351,53 @@ int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmLaunch& l, hipStream_
   magic_divisor(chunk_divisor, &ka.m_chunks, &ka.s_chunks);
   magic_divisor((uint32_t)l.tile_split, &ka.m_colblocks, &ka.s_colblocks);
   if (l.lockstep_log2 >= 0) ka.s_colblocks = (uint32_t)l.lockstep_log2;
-  magic_divisor((uint32_t)a.ngroups, &ka.m_ngroups, &ka.s_ngroups);
-  if (l.packed_log2 >= 0) ka.m_ngroups = (uint32_t)(a.tiles_h * a.tiles_w);  // the spatial tiles
+  magic_divisor((uint32_t)(l.packed ? a.N : a.ngroups), &ka.m_ngroups, &ka.s_ngroups);
   magic_divisor((uint32_t)a.tiles_w, &ka.m_tiles_w, &ka.s_tiles_w);
   size_t ka_size = sizeof(ka);
   void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &ka, HIP_LAUNCH_PARAM_BUFFER_SIZE, &ka_size,
                    HIP_LAUNCH_PARAM_END};
-  return (int)hipModuleLaunchKernel(l.fn, (unsigned)grid, 1, 1, 256, 1, 1, (unsigned)l.lds_bytes, st,
-                                    nullptr, extra);
+  const hipError_t e = hipModuleLaunchKernel(l.fn, (unsigned)grid, 1, 1, 256, 1, 1, (unsigned)l.lds_bytes,
+                                             st, nullptr, extra);
+  if (e == hipSuccess) t_last_kernel = l.name;
+  return (int)e;
 }
 
-// Batches of 16 and fewer: the assembly kernels fill the 32 columns of a column tile with
-// NB = 2^k >= N batch elements of 32 / NB consecutive spatial tiles (_packed kernels) instead of
-// leaving columns empty.  Returns log2 NB, or -1 for larger batches; *a gets the packed column
-// tiles.
-int pack_columns(opencnn::ConvArgs* a) {
-  if (a->N > 16) return -1;
-  int log2nb = 0;
-  while ((1 << log2nb) < a->N) ++log2nb;
-  const int per_tile = 32 >> log2nb;
+// Batches that are no multiple of 32: the _packed assembly kernels put the columns of all
+// (spatial tile, batch element) pairs on one line and cut it into column tiles of 32, so only the
+// last column tile has empty columns.  A packed column tile costs 5-8 % more (its lanes' loads
+// straddle two spatial tiles), so: only when an eighth or more of the columns would be empty, and
+// when the unpacked layer (unpacked_tiles workgroup tiles) has more than one round of tiles for
+// the compute units - a layer that fits one round takes one tile's time either way.
+// Returns whether the shape is packed; *a then holds the packed column tiles.
+int pack_columns(opencnn::ConvArgs* a, long long unpacked_tiles, bool* packed) {
+  *packed = false;
+  if (a->N % 32 == 0 || a->N * 8 > a->ngroups * 32 * 7) return 0;
+  int cus = 0;
+  if (int e = compute_units(&cus)) return e;
+  if (unpacked_tiles <= cus) return 0;
+  const long long columns = (long long)a->tiles_h * a->tiles_w * a->N;  // below 2^31: it divides the output
   a->ngroups = 1;
-  a->colgroups = (a->tiles_h * a->tiles_w + per_tile - 1) / per_tile;
-  return log2nb;
+  a->colgroups = (int)((columns + 31) / 32);
+  *packed = true;
+  return 0;
 }
 
-int launch_asm(const opencnn::ConvArgs& a, int kw, int grid, bool ragged, int packed_log2, size_t lds_bytes,
+int launch_asm(const opencnn::ConvArgs& a, int kw, int grid, bool ragged, bool packed, size_t lds_bytes,
                hipStream_t st) {
   const AsmKernels* ak = nullptr;
   if (int e = asm_kernels(&ak)) return e;
   AsmLaunch l;
-  if (packed_log2 >= 0)
+  if (packed) {
     l.fn = kw == 4 ? ak->kw4_packed : ak->kw2_packed;
-  else
-    l.fn = ragged ? (kw == 4 ? ak->kw4_ragged : ak->kw2_ragged) : (kw == 4 ? ak->kw4 : ak->kw2);
-  l.packed_log2 = packed_log2;
+    l.name = kw == 4 ? "wino_f32_asm_kw4_packed" : "wino_f32_asm_kw2_packed";
+  } else if (ragged) {
+    l.fn = kw == 4 ? ak->kw4_ragged : ak->kw2_ragged;
+    l.name = kw == 4 ? "wino_f32_asm_kw4_ragged" : "wino_f32_asm_kw2_ragged";
+  } else {
+    l.fn = kw == 4 ? ak->kw4 : ak->kw2;
+    l.name = kw == 4 ? "wino_f32_asm_kw4" : "wino_f32_asm_kw2";
+  }
+  l.packed = packed;
   l.grid = grid;
   l.lds_bytes = lds_bytes;
   l.chunks = (a.C + 7) / 8;
@@ -393,7 +415,8 @@ constexpr int kEpilogueHalfUnits = 3;
 
 int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* launched) {
   *launched = false;
-  const int packed_log2 = pack_columns(&a);
+  bool packed = false;
+  if (int e = pack_columns(&a, (long long)a.colgroups * ((a.kgroups + 3) / 4), &packed)) return e;
   // Any shape.  Waves of the last filter block whose 32 filters do not exist help with the input
   // transform, multiply zeros and store nothing.  In the _ragged kernels the last chunk's missing
   // channels read as zeros (descriptor cut at the tensor's end) and meet zero rows of the padded
@@ -414,11 +437,14 @@ int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* lau
   AsmLaunch l;
   // the _ragged kernels mask batch elements, channels and filter rows that do not exist
   const bool ragged = a.N % 32 != 0 || a.C % 16 != 0 || a.K % 32 != 0;
-  if (precision == OPENCNN_BF16)
-    l.fn = packed_log2 >= 0 ? ak->bf16_kw4_packed : (ragged ? ak->bf16_kw4_ragged : ak->bf16_kw4);
-  else
-    l.fn = packed_log2 >= 0 ? ak->f16_kw4_packed : (ragged ? ak->f16_kw4_ragged : ak->f16_kw4);
-  l.packed_log2 = packed_log2;
+  if (precision == OPENCNN_BF16) {
+    l.fn = packed ? ak->bf16_kw4_packed : (ragged ? ak->bf16_kw4_ragged : ak->bf16_kw4);
+    l.name = packed ? "wino_bf16_asm_kw4_packed" : (ragged ? "wino_bf16_asm_kw4_ragged" : "wino_bf16_asm_kw4");
+  } else {
+    l.fn = packed ? ak->f16_kw4_packed : (ragged ? ak->f16_kw4_ragged : ak->f16_kw4);
+    l.name = packed ? "wino_f16_asm_kw4_packed" : (ragged ? "wino_f16_asm_kw4_ragged" : "wino_f16_asm_kw4");
+  }
+  l.packed = packed;
   l.grid = grid;
   l.lds_bytes = 2 * 16 * 2 * 4 * 32 * sizeof(unsigned);  // two buffers of V
   l.chunks = chunks;
@@ -454,14 +480,14 @@ int launch_hip(const opencnn::ConvArgs& a, int kw, bool ragged, bool allow_strea
       opencnn::wino_f32_fused<true><<<grid, block, 0, st>>>(a);
     else
       opencnn::wino_f32_fused<false><<<grid, block, 0, st>>>(a);
-    return (int)hipGetLastError();
+    return launched_hip("wino_f32_fused");
   }
   if (ragged) {
     if (kw == 4)
       opencnn::wino_f32_fused_lds<4, false, true><<<grid, block, lds_bytes, st>>>(a);
     else
       opencnn::wino_f32_fused_lds<2, false, true><<<grid, block, lds_bytes, st>>>(a);
-    return (int)hipGetLastError();
+    return launched_hip("wino_f32_fused_lds");
   }
   // More tiles than CUs and not a whole number of rounds: one persistent workgroup per CU,
   // the chunk-units split evenly (every tile then has at most two contributors).
@@ -489,7 +515,7 @@ int launch_hip(const opencnn::ConvArgs& a, int kw, bool ragged, bool allow_strea
     else
       opencnn::wino_f32_fused_lds<2, false><<<grid, block, lds_bytes, st>>>(a);
   }
-  return (int)hipGetLastError();
+  return launched_hip(stream ? "wino_f32_stream" : "wino_f32_fused_lds");
 }
 
 int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c, int in_h,
@@ -548,12 +574,14 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
     // is faster there (measured, K = 32).
     const int kw = a.kgroups == 1 ? 1 : ((a.kgroups + 3) / 4 * 4 <= (a.kgroups + 1) / 2 * 2 ? 4 : 2);
     opencnn::ConvArgs b = a;
-    const int packed_log2 = pack_columns(&b);
+    REQUIRE(tile_with(b, kw));
+    bool packed = false;
+    if (int e = pack_columns(&b, b.nblocks, &packed)) return e;
     REQUIRE(tile_with(b, kw));
     int grid = 0;
     if (int e = asm_grid(b, kw, (b.C + 7) / 8, &grid)) return e;
     if (grid > 0)
-      return launch_asm(b, kw, grid, ragged || b.kgroups % kw != 0, packed_log2, lds_bytes(kw), st);
+      return launch_asm(b, kw, grid, ragged || b.kgroups % kw != 0, packed, lds_bytes(kw), st);
     REQUIRE(variant != OPENCNN_KERNEL_ASM);
   }
   // The HIP C++ kernels: as many sharing waves as the (rounded-up) filter groups fill whole
@@ -570,6 +598,8 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
 extern "C" {
 
 const char* opencnn_last_error(void) { return t_last_error; }
+
+const char* opencnn_last_kernel(void) { return t_last_kernel; }
 
 int opencnn_init(void) {
   int dev = 0;

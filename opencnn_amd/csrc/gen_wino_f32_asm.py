@@ -96,8 +96,8 @@ class Kernel:
         self.ragged = ragged
         # batch elements, and filters, that do not exist are masked (the fp16 / bf16 kernels always do)
         self.ragged_n = self.ragged_k = ragged
-        # packed (batches of 16 and fewer, a _ragged kernel): the 32 columns of a column tile are
-        # NB = 2^k >= N batch elements of 32 / NB consecutive spatial tiles; see lane_tile
+        # packed (batches that are no multiple of 32, a _ragged kernel): a column tile is 32
+        # consecutive columns of the line of all (spatial tile, batch element) pairs; see lane_tile
         self.packed = packed
         self.CW = 4 // KW
         self.SPW = 4 // KW
@@ -252,30 +252,34 @@ class Kernel:
             if i < 3:
                 self.e(f"s_add_i32 {t(2)}, {t(2)}, {self.sr('RowStep')}")
 
-    # ------------------------------------------------------------------ packed column tiles (N <= 16)
-    # Column n32 of column tile g: batch element n32 & (NB - 1) of spatial tile g * (32 / NB) +
-    # (n32 >> log2 NB), tiles numbered row-major.  The argument slot Ngroups carries log2 NB, the
-    # slot Mng the number of spatial tiles.  Everything per lane happens here, at a tile switch:
-    # the units only see 16 patch offsets and 4 store offsets per lane, as before.  Scratch: the
-    # transform temporaries T, dead between two units.
+    # ------------------------------------------------------------------ packed column tiles (N % 32 != 0)
+    # The columns of all spatial tiles (numbered row-major) and their N batch elements form one
+    # line, column (tile, n) at tile * N + n; column tile g holds columns 32 g .. 32 g + 31 of it,
+    # so only the last column tile of a layer has empty columns.  The magic number of the slot
+    # Mng / Sng divides by N.  Everything per lane happens here, at a tile switch: the units only
+    # see 16 patch offsets and 4 store offsets per lane, as before.  Scratch: the transform
+    # temporaries T, dead between two units.
     def lane_tile(self):
-        """T[0] = batch element, T[1] = 2*ty, T[2] = 2*tx of this lane's tile in column tile Dty;
-        T[3] = 0, or the out-of-range bit for a lane whose tile or batch element does not exist."""
+        """T[0] = batch element * 4, T[1] = 2*ty, T[2] = 2*tx of this lane's column in column tile
+        Dty; T[3] = 0, or the out-of-range bit for a lane past the last column."""
         t = self.t
         T = lambda i: self.vr("T", i)
         self.e(f"v_and_b32 {T(0)}, 31, {self.vr('Lane')}")
-        self.e(f"v_lshrrev_b32 {T(1)}, {self.sr('Ngroups')}, {T(0)}")       # tile within the group
-        self.e(f"s_lshl_b32 {t(4)}, 1, {self.sr('Ngroups')}")
-        self.e(f"s_sub_u32 {t(4)}, {t(4)}, 1")
-        self.e(f"v_and_b32 {T(0)}, {t(4)}, {T(0)}")                         # batch element
-        self.e(f"s_lshr_b32 {t(4)}, 32, {self.sr('Ngroups')}")
-        self.e(f"s_mul_i32 {t(4)}, {t(4)}, {self.sr('Dty')}")
-        self.e(f"v_add_u32 {T(1)}, {t(4)}, {T(1)}")                         # spatial tile
-        self.e(f"v_cmp_gt_u32 vcc, {self.sr('Mng')}, {T(1)}")               # it exists
+        self.e(f"s_lshl_b32 {t(4)}, {self.sr('Dty')}, 5")
+        self.e(f"v_add_u32 {T(1)}, {t(4)}, {T(0)}")                         # column on the line
+        # tile = column / N with the magic number, in 64 bits as the scalar div does
+        self.e(f"v_mul_lo_u32 {T(4)}, {T(1)}, {self.sr('Mng')}")
+        self.e(f"v_mul_hi_u32 {T(5)}, {T(1)}, {self.sr('Mng')}")
+        self.e(f"v_lshrrev_b64 {self.vr('T', 4, 2)}, {self.sr('Sng')}, {self.vr('T', 4, 2)}")
+        self.e(f"v_mul_lo_u32 {T(5)}, {T(4)}, {self.sr('N')}")
+        self.e(f"v_sub_u32 {T(0)}, {T(1)}, {T(5)}")                         # batch element
+        self.e(f"v_mov_b32 {T(1)}, {T(4)}")                                 # spatial tile
+        self.e(f"s_add_u32 {t(4)}, {self.sr('H')}, 1")
+        self.e(f"s_lshr_b32 {t(4)}, {t(4)}, 1")
+        self.e(f"s_mul_i32 {t(4)}, {t(4)}, {self.sr('TilesW')}")
+        self.e(f"v_cmp_gt_u32 vcc, {t(4)}, {T(1)}")                         # the tile exists
         self.e(f"v_cndmask_b32 {T(3)}, {self.vr('Oob')}, {self.vr('Zero')}, vcc")
-        self.e(f"v_cmp_le_u32 vcc, {self.sr('N')}, {T(0)}")                 # the batch element does not
-        self.e(f"v_cndmask_b32 {T(3)}, {T(3)}, {self.vr('Oob')}, vcc")
-        # ty = tile / TilesW with the magic number, in 64 bits as the scalar div does
+        # ty = tile / TilesW
         self.e(f"v_mul_lo_u32 {T(4)}, {T(1)}, {self.sr('Mtw')}")
         self.e(f"v_mul_hi_u32 {T(5)}, {T(1)}, {self.sr('Mtw')}")
         self.e(f"v_lshrrev_b64 {self.vr('T', 4, 2)}, {self.sr('Stw')}, {self.vr('T', 4, 2)}")

@@ -58,7 +58,7 @@ class KernelH16(Kernel):
     def __init__(self, bf16, ragged=False, packed=False):
         """ragged: shapes outside N % 32 == 0, C % 16 == 0, K % 32 == 0 (masked lanes and rows, a
         slab descriptor that ends with the tensor; a few scalar instructions per unit and row).
-        packed: a _ragged kernel for batches of 16 and fewer (Kernel.lane_tile)."""
+        packed: a _ragged kernel for batches that are no multiple of 32 (Kernel.lane_tile)."""
         self.bf16 = bf16
         self.KW, self.CW, self.SPW = 4, 1, 1
         self.ragged = False  # the fp32 kernels' two-channel slab logic is replaced, see slab_descriptor

@@ -121,6 +121,9 @@ def test_benchmark_configs(ocn, oracle, torch_gpu, name, N, C, H, K, xr, filt):
     print(f"config {name} N={N} C={C} H={H} K={K}", flush=True)
     x, w = make_tensors(ocn, N, C, H, H, K, xr, filt)
     y = Runner(ocn, torch_gpu, x, w).dropin()
+    # the default choice on the benchmark layers is a hand-scheduled kernel (K = 64: two waves
+    # share a column tile, else four)
+    assert ocn.last_kernel() == ("wino_f32_asm_kw2" if K == 64 else "wino_f32_asm_kw4")
     rel, rel64 = check_against_oracle(oracle, y, x, w)
     print(f"  rel-L2 vs Winograd restatement {rel:.2e}, vs fp64 direct {rel64:.2e}", flush=True)
 
@@ -356,6 +359,7 @@ def test_benchmark_configs_on_hip_kernels(ocn, oracle, torch_gpu, name, N, C, H,
     try:
         ocn.set_kernel_variant(ocn.KERNEL_HIP)
         y = Runner(ocn, torch_gpu, x, w).dropin()
+        assert ocn.last_kernel() in ("wino_f32_fused_lds", "wino_f32_stream")
     finally:
         ocn.set_kernel_variant(ocn.KERNEL_AUTO)
     check_against_oracle(oracle, y, x, w)
@@ -410,15 +414,23 @@ def test_buffers_need_only_float_alignment(ocn, oracle, torch_gpu, family, prec,
         assert rel <= (1e-5 if prec == "f32" else 2e-3), f"rel-L2 vs fp64 direct {rel:.3e}"
 
 
-# batches of 16 and fewer: the assembly kernels pack several spatial tiles into a column tile
-PACKED_SHAPES = [(1, 64, 14, 14, 64), (2, 16, 7, 9, 128), (3, 8, 5, 5, 64), (4, 32, 28, 28, 96),
-                 (5, 24, 13, 17, 100), (8, 256, 14, 14, 256), (9, 40, 6, 6, 250), (16, 64, 56, 56, 64),
-                 (16, 8, 1, 1, 64), (7, 3, 33, 20, 40), (1, 16, 112, 112, 64), (12, 20, 2, 3, 160)]
+# batches that are no multiple of 32: the assembly kernels cut their column tiles from the line of
+# all (spatial tile, batch element) pairs, so a column tile holds several tiles or parts of two.
+# The library packs when an eighth of the columns would be empty and the layer has more workgroup
+# tiles than compute units; the last four shapes stay on the unpacked _ragged kernels.
+PACKED_SHAPES = [(1, 8, 64, 64, 64, True), (2, 16, 47, 39, 128, True), (3, 8, 45, 45, 64, True),
+                 (5, 24, 33, 37, 100, True), (7, 3, 41, 50, 40, True), (9, 40, 36, 36, 250, True),
+                 (12, 20, 40, 30, 160, True), (16, 64, 56, 56, 64, True), (17, 16, 50, 50, 64, True),
+                 (20, 8, 36, 44, 128, True), (33, 24, 23, 23, 96, True), (40, 16, 28, 28, 128, True),
+                 (48, 32, 40, 40, 64, True), (100, 128, 28, 28, 128, True), (70, 8, 30, 30, 64, True),
+                 (1, 16, 112, 112, 64, True),
+                 (1, 64, 14, 14, 64, False), (8, 256, 14, 14, 256, False), (60, 8, 40, 40, 64, False),
+                 (127, 16, 25, 25, 256, False)]
 
 
 @pytest.mark.parametrize("prec", ["f32", "f16", "bf16"])
-@pytest.mark.parametrize("N,C,H,W,K", PACKED_SHAPES)
-def test_small_batches_on_packed_column_tiles(ocn, oracle, torch_gpu, prec, N, C, H, W, K):
+@pytest.mark.parametrize("N,C,H,W,K,packed", PACKED_SHAPES)
+def test_batches_on_packed_column_tiles(ocn, oracle, torch_gpu, prec, N, C, H, W, K, packed):
     # the assembly kernels selected explicitly; against the fp64 direct convolution, the HIP C++
     # kernels (which leave the columns of missing batch elements empty) and a second call
     print(f"packed {prec} N={N} C={C} H={H} W={W} K={K}", flush=True)
@@ -428,12 +440,16 @@ def test_small_batches_on_packed_column_tiles(ocn, oracle, torch_gpu, prec, N, C
         ocn.set_operand_precision({"f32": ocn.F32, "f16": ocn.F16, "bf16": ocn.BF16}[prec])
         ocn.set_kernel_variant(ocn.KERNEL_ASM)
         y = r.split()
+        kernel = ocn.last_kernel()
         y2 = r.split()
         ocn.set_kernel_variant(ocn.KERNEL_HIP)
         y_hip = r.split()
+        assert "_asm_" not in ocn.last_kernel()
     finally:
         ocn.set_kernel_variant(ocn.KERNEL_AUTO)
         ocn.set_operand_precision(ocn.F32)
+    assert kernel.startswith(f"wino_{prec}_asm_kw")
+    assert kernel.endswith("_packed" if packed else "_ragged"), kernel
     assert not np.isnan(y).any(), "an output element was never written"
     assert np.array_equal(y, y2)
     bound = {"f32": 1e-5, "f16": 2e-3, "bf16": 1.5e-2}[prec]
