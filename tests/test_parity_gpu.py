@@ -509,18 +509,27 @@ def test_ragged_shape_on_every_kernel_family(ocn, oracle, torch_gpu, N, C, H, K)
         ocn.set_kernel_variant(ocn.KERNEL_AUTO)
 
 
-def test_padded_channels_do_not_leak_non_finite_values(ocn, oracle, torch_gpu):
-    # C = 5 runs one 8-channel chunk; the three padded channels multiply zeros on BOTH operands,
-    # so an infinity in the last real channel must stay confined to the outputs it reaches
-    print("ragged inf", flush=True)
-    for K in (32, 64):  # register kernel / assembly kernel
-        N, C, H = 32, 5, 6
+@pytest.mark.parametrize("prec", ["f32", "f16", "bf16"])
+def test_padded_channels_do_not_leak_non_finite_values(ocn, oracle, torch_gpu, prec):
+    # C = 5 runs one chunk of 8 (fp16 / bf16: 16) channels; the padded channels multiply zeros on
+    # BOTH operands, so an infinity in the last real channel must stay confined to the outputs it
+    # reaches: the batch element it sits in
+    print(f"ragged inf {prec}", flush=True)
+    # K = 32: register kernel (fp32); K = 64: assembly kernel; N = 3 on 40x40: packed column tiles,
+    # where the lanes next to the infinity's belong to other spatial tiles
+    for N, H, K, n_inf in ((32, 6, 32, 3), (32, 6, 64, 3), (3, 40, 64, 1)):
+        C = 5
         x, w = make_tensors(ocn, N, C, H, H, K, filt="uniform")
-        x[C - 1, 2, 2, 3] = np.inf
-        y = Runner(ocn, torch_gpu, x, w).split()
+        x[C - 1, 2, 2, n_inf] = np.inf
+        try:
+            ocn.set_operand_precision({"f32": ocn.F32, "f16": ocn.F16, "bf16": ocn.BF16}[prec])
+            y = Runner(ocn, torch_gpu, x, w).split()
+        finally:
+            ocn.set_operand_precision(ocn.F32)
         bad = ~np.isfinite(y)
-        assert bad[:, :, :, 3].any()
-        bad[:, :, :, 3] = False
+        assert bad[:, :, :, n_inf].any()
+        assert not bad[:, 5:, :, n_inf].any() and not bad[:, :, 5:, n_inf].any()  # a 3x3 filter's reach
+        bad[:, :, :, n_inf] = False
         assert not bad.any()
 
 
