@@ -196,8 +196,8 @@ int launch_fx(const float* w, float* Ww, int filt_k, int filt_c, int filter_layo
   const int precision = g_precision.load();
   if (ww_layout == OPENCNN_WW_MFMA && precision != OPENCNN_F32) {
     // padded to whole pairs of 32-wide filter groups and 16-channel chunks, zeros in the padding
-    dim3 grid((unsigned)((padded_k_h16(filt_k) + 127) / 128), (unsigned)(padded_c_h16(filt_c) / 16)), block(256);
-    uint4* out = reinterpret_cast<uint4*>(Ww);
+    dim3 grid((unsigned)(padded_k_h16(filt_k) / 64), (unsigned)(padded_c_h16(filt_c) / 16)), block(256);
+    uint2* out = reinterpret_cast<uint2*>(Ww);
     if (precision == OPENCNN_F16) {
       if (kcrs)
         opencnn::fx_mfma_layout_h16<true, false><<<grid, block, 0, st>>>(w, out, filt_k, filt_c);

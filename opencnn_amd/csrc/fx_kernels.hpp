@@ -104,8 +104,8 @@ __global__ void __launch_bounds__(256) fx_mfma_layout(const float* __restrict__ 
 //   Uh[kg][chunk][p][h][k32][e] (2-byte elements),  k = kg*32 + k32,  c = 16*chunk + 8*h + e
 // so that lane (h*32 + k32) of a wave fetches, with one 16-byte load per position p, the A
 // operand of one v_mfma_f32_32x32x16_{f16,bf16} (16 input channels).  U is computed in fp32 in
-// the reference's order and rounded to nearest-even once.  Thread = (k, chunk, h).
-// grid (ceil(Kpad/128), ceil(C/16)), block 256 = 2 h x 128 k.  The layout covers
+// the reference's order and rounded to nearest-even once.
+// grid (Kpad/64, ceil(C/16)), block 256 = 64 k x 2 h x 2 halves of 4 channels.  The layout covers
 // Kpad = 64*ceil(K/64) filters (whole pairs of 32-wide groups, the smallest workgroup of the
 // fused kernel) and 16*ceil(C/16) channels; filters / channels that do not exist are zeros.
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
@@ -119,17 +119,20 @@ __device__ __forceinline__ unsigned pack_pair(float lo, float hi) {
   return __builtin_bit_cast(unsigned, __builtin_convertvector(f, v2h));
 }
 
+// One thread: filter k, four consecutive channels (a quarter of a 16-channel chunk), all 16
+// positions; 8 bytes per position of the lane's 16-byte MFMA operand.  A workgroup covers 64
+// filters of one chunk.
 template <bool KCRS, bool BF16>
 __global__ void __launch_bounds__(256) fx_mfma_layout_h16(const float* __restrict__ w,
-                                                          uint4* __restrict__ Uh, int K, int C) {
-  const int h = threadIdx.x >> 7;
-  const int k = blockIdx.x * 128 + (threadIdx.x & 127);
+                                                          uint2* __restrict__ Uh, int K, int C) {
+  const int k = blockIdx.x * 64 + (threadIdx.x & 63);
+  const int h = (threadIdx.x >> 6) & 1;   // which 8 channels of the chunk: the operand's lane half
+  const int half = threadIdx.x >> 7;      // which 4 of those 8
   const int chunk = blockIdx.y;
-  if (k >= ((K + 63) & ~63)) return;
-  float U[8][16];
+  float U[4][16];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const int c = 16 * chunk + 8 * h + e;
+  for (int e = 0; e < 4; ++e) {
+    const int c = 16 * chunk + 8 * h + 4 * half + e;
     if (k < K && c < C) {
       float g[9];
       load_filter<KCRS>(w, c, k, C, K, g);
@@ -140,11 +143,10 @@ __global__ void __launch_bounds__(256) fx_mfma_layout_h16(const float* __restric
     }
   }
   const int kg = k >> 5, k32 = k & 31;
-  uint4* o = Uh + (((size_t)kg * gridDim.y + chunk) * 16) * 64 + h * 32 + k32;
+  uint2* o = Uh + ((((size_t)kg * gridDim.y + chunk) * 16) * 64 + h * 32 + k32) * 2 + half;
 #pragma unroll
   for (int p = 0; p < 16; ++p)
-    o[(size_t)p * 64] = make_uint4(pack_pair<BF16>(U[0][p], U[1][p]), pack_pair<BF16>(U[2][p], U[3][p]),
-                                   pack_pair<BF16>(U[4][p], U[5][p]), pack_pair<BF16>(U[6][p], U[7][p]));
+    o[(size_t)p * 128] = make_uint2(pack_pair<BF16>(U[0][p], U[1][p]), pack_pair<BF16>(U[2][p], U[3][p]));
 }
 
 }  // namespace opencnn
