@@ -162,7 +162,10 @@ int opencnn_set_kernel_variant(int variant);
  * 3.06 rounds, which plain launching rounds up to 4), one persistent workgroup per CU takes an
  * equal share of (tile, 8-channel chunk) units; a tile whose channel range ends up split
  * between two workgroups is merged through the output tensor and two words of library-owned
- * device state per wave.  Results stay independent of timing (two addends commute).  That
+ * device state per wave.  Results stay independent of timing (two addends commute).  The same
+ * hand-over serves layers with tiles for at most half of the compute units (small batches on
+ * deep layers, fp32 operands): every tile is cut among two or four workgroups, and the parts of
+ * its channel sum are passed from workgroup to workgroup in a fixed order.  That
  * state exists once per stream for the first eight streams that launch (calls on different
  * streams may overlap in time); calls on further streams run without the split.  Pass 0 to
  * turn it off altogether.  No counterpart in the reference, whose grid is one block per tile

@@ -271,18 +271,36 @@ int launch_h16(opencnn::ConvArgs a, int precision, hipStream_t st) {
 // Grid of the hand-scheduled kernels for this layer, or 0 when they do not take it.  One
 // persistent launch whose workgroups share the (tile, chunk) units evenly; it needs whole filter
 // blocks (kw > 1) and at least one tile per workgroup (a tile then has at most two contributors).
-int asm_grid(const opencnn::ConvArgs& a, int kw, int chunks, int* grid) {
+// A layer with tiles for at most half of the compute units: every tile is cut into `pieces`
+// equal runs of units, one workgroup each.  The last piece publishes its part of the outputs,
+// every other one adds the part published behind it in its output transform and publishes the
+// sum, the first stores the tile: a chain of pieces - 1 hand-overs of about 5 us behind
+// 1 / pieces of the tile's units.  Pieces of at least kMinUnitsPerPiece units.
+constexpr int kMinUnitsPerPiece = 8;
+
+int pieces_per_tile(int nblocks, int chunks, int cus) {
+  int pieces = 1;
+  while (pieces < 4 && nblocks * pieces * 2 <= cus && nblocks * pieces * 2 <= opencnn::kMaxBalancedBlocks &&
+         chunks % (pieces * 2) == 0 && chunks / (pieces * 2) >= kMinUnitsPerPiece)
+    pieces *= 2;
+  return pieces;
+}
+
+// cut_tiles: the kernel can merge in its output transform (the fp32 kernels).
+int asm_grid(const opencnn::ConvArgs& a, int kw, int chunks, bool cut_tiles, int* grid) {
   *grid = 0;
   if (kw == 1 || (long long)a.nblocks * chunks > kMaxElems) return 0;
   // per-lane store offsets: four filter rows plus one image row and column, in bytes
   if (((long long)a.N * a.H * a.W * 4 + (long long)(a.W + 1) * a.N) * 4 > kMaxElems) return 0;
   int cus = 0;
   if (int e = compute_units(&cus)) return e;
-  if (a.nblocks < cus)
+  const bool split = g_balance.load() != 0 && a.sync != nullptr;
+  if (a.nblocks < cus) {
     *grid = a.nblocks;  // one tile per workgroup
-  else if (cus % 8 == 0 && cus <= opencnn::kMaxBalancedBlocks &&
-           (a.nblocks % cus == 0 || (g_balance.load() != 0 && a.sync != nullptr)))
+    if (cut_tiles && split) *grid = a.nblocks * pieces_per_tile(a.nblocks, chunks, cus);
+  } else if (cus % 8 == 0 && cus <= opencnn::kMaxBalancedBlocks && (a.nblocks % cus == 0 || split)) {
     *grid = cus;
+  }
   return 0;
 }
 
@@ -430,7 +448,8 @@ int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* lau
   a.nblocks = (int)nblocks;
   a.colblocks = a.colgroups;
   int grid = 0;
-  if (int e = asm_grid(a, 4, chunks, &grid)) return e;
+  // (tiles are not cut: these kernels cannot merge in their output transform)
+  if (int e = asm_grid(a, 4, chunks, false, &grid)) return e;
   if (grid == 0) return 0;
   const AsmKernels* ak = nullptr;
   if (int e = asm_kernels(&ak)) return e;
@@ -579,7 +598,7 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
     if (int e = pack_columns(&b, b.nblocks, &packed)) return e;
     REQUIRE(tile_with(b, kw));
     int grid = 0;
-    if (int e = asm_grid(b, kw, (b.C + 7) / 8, &grid)) return e;
+    if (int e = asm_grid(b, kw, (b.C + 7) / 8, true, &grid)) return e;
     if (grid > 0)
       return launch_asm(b, kw, grid, ragged || b.kgroups % kw != 0, packed, lds_bytes(kw), st);
     REQUIRE(variant != OPENCNN_KERNEL_ASM);

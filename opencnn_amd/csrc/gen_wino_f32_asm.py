@@ -657,14 +657,17 @@ class Kernel:
         if self.ragged_k:
             self.row_limit(r + 1)
 
-    def epilogue(self, through):
+    def epilogue(self, through, merge=False):
         """Y = A^T M A per accumulator element (order of src/store_and_transform_output_optSTS64.cuh:29-51)
         and the 64 stores of the tile; `through` = write past the caches (a partial tile that a
-        workgroup on another XCD will read)."""
+        workgroup on another XCD will read).  `merge`: the partial tile that the next workgroup
+        published is added to the outputs here (late_merge)."""
         # final outputs are written once and never read again by this kernel: non-temporal, so that
         # they do not push the input patches that neighbouring tiles share out of L2
         pol = " sc0 sc1" if through else " nt"
         ry = self.S["RsrcY"]
+        if merge:
+            land = self.late_merge_loads()
         self.row_start()
         # the last MFMAs must have written the accumulators before they are read
         self.e("s_nop 15")
@@ -694,6 +697,12 @@ class Kernel:
             self.e(f"v_sub_f32 {o(1)}, {o(1)}, {w(3)}")
             self.e(f"v_add_f32 {o(2)}, {o(2)}, {w(6)}")
             self.e(f"v_sub_f32 {o(3)}, {o(3)}, {w(7)}")
+            if merge:
+                if r == 0:
+                    self.e("s_waitcnt vmcnt(0)")  # the partial tile has landed (no store is out yet)
+                    self.store_flag(self.vr("Zero"))  # hand the flag back for the next launch
+                for q in range(4):
+                    self.e(f"v_add_f32 {o(q)}, {o(q)}, {v(land[r * 4 + q])}")
             pending = [f"buffer_store_dword {o(q)}, {self.vr('Eff', q)}, {s(ry, 4)}, 0 offen{pol}" for q in range(4)]
             if r == 15:
                 for st in pending:
@@ -716,12 +725,9 @@ class Kernel:
         self.e(f"global_store_dword {self.vr('Zero')}, {value_reg}, {s(self.S['Fl'], 2)} sc0 sc1")
         self.e("s_mov_b64 exec, -1")
 
-    def merge_init(self):
-        """Last segment of a workgroup that ends inside a tile: the first part of that tile was
-        published by the next workgroup long ago.  Wait for its flag (bounded), read the partial
-        outputs past the caches and start the accumulators from them."""
+    def wait_flag(self):
+        """Until the workgroup behind this one has published its part of the tile (bounded)."""
         t = self.t
-        self.comment("---- merge: accumulators start from the published partial tile")
         self.flag_address(False)
         self.e(f"s_mov_b32 {self.sr('Spin')}, 0")
         poll, got = self.newlabel("poll"), self.newlabel("got")
@@ -738,6 +744,35 @@ class Kernel:
         self.e("s_sleep 8")
         self.e(f"s_branch {poll}")
         self.label(got)
+
+    def late_merge_registers(self):
+        """64 registers for a partial tile that is added in the output transform.  That transform is
+        the last thing its workgroup does, so the filter registers are dead; a prefetch into them
+        that is still in flight lands before the partial tile (loads return in order)."""
+        return [self.V["U0"] + i for i in range(32)] + [self.V["U1"] + i for i in range(32)]
+
+    def late_merge_loads(self):
+        """A range that lies inside one tile (a layer with few tiles, cut among several
+        workgroups): every workgroup of the tile finishes its units at the same time, so the
+        published part of the tile cannot be in the accumulators before the first unit as in
+        merge_init.  Wait for it here and add it to the outputs (epilogue)."""
+        land = self.late_merge_registers()
+        ry = self.S["RsrcY"]
+        self.comment("---- late merge: the partial tile is added in the output transform")
+        self.wait_flag()
+        self.row_start()
+        for r in range(16):
+            for q in range(4):
+                self.e(f"buffer_load_dword {v(land[r * 4 + q])}, {self.vr('Eff', q)}, {s(ry, 4)}, 0 offen sc0 sc1")
+            self.row_advance(r)
+        return land
+
+    def merge_init(self):
+        """Last segment of a workgroup that ends inside a tile: the first part of that tile was
+        published by the next workgroup long ago.  Wait for its flag (bounded), read the partial
+        outputs past the caches and start the accumulators from them."""
+        self.comment("---- merge: accumulators start from the published partial tile")
+        self.wait_flag()
         ry = self.S["RsrcY"]
         self.row_start()
         for r in range(16):
@@ -942,7 +977,11 @@ class Kernel:
         e(f"s_cselect_b32 {self.sr('Kind')}, 1, 0")
         e(f"s_cmp_lt_u32 {self.sr('SegEnd')}, {self.sr('Chunks')}")
         e(f"s_cbranch_scc0 {plain_seg}")
-        e(f"s_mov_b32 {self.sr('Kind')}, 2")
+        # a range shorter than a tile: the merge waits until the output transform (Kind 4 and 5)
+        e(f"s_or_b32 {t(0)}, {self.sr('Kind')}, 4")
+        e(f"s_cmp_lt_u32 {self.sr('Nunits')}, {self.sr('Chunks')}")
+        e(f"s_cselect_b32 {self.sr('Kind')}, {t(0)}, 2")
+        e(f"s_cbranch_scc1 {plain_seg}")
         self.merge_init()
         self.chunk("merge")
         e(f"s_branch {check}")
@@ -957,13 +996,16 @@ class Kernel:
         e(f"s_cbranch_scc1 {regular}")
         self.label(epi_plain)
         self.stamp()
-        pub = self.newlabel("publish")
+        pub, late, late_pub, flag = (self.newlabel(x) for x in ("publish", "late", "latepub", "flag"))
         e(f"s_cmp_eq_u32 {self.sr('Kind')}, 1")
         e(f"s_cbranch_scc1 {pub}")
+        e(f"s_cmp_ge_u32 {self.sr('Kind')}, 4")
+        e(f"s_cbranch_scc1 {late}")
         self.epilogue(False)
         e(f"s_branch {after_epi}")
         self.label(pub)
         self.epilogue(True)
+        self.label(flag)
         e("s_waitcnt vmcnt(0)")  # every write-through store acknowledged, then the flag
         self.flag_address(True)
         self.store_flag(self.vr("One"))
@@ -979,6 +1021,15 @@ class Kernel:
         e(f"s_branch {seg_loop}")
         self.label(done)
         e("s_endpgm")
+        # the output transforms with a late merge (layers with few tiles only)
+        self.label(late)
+        e(f"s_cmp_eq_u32 {self.sr('Kind')}, 5")
+        e(f"s_cbranch_scc1 {late_pub}")
+        self.epilogue(False, merge=True)
+        e(f"s_branch {after_epi}")
+        self.label(late_pub)
+        self.epilogue(True, merge=True)
+        e(f"s_branch {flag}")
         self.lines.extend(self.outofline)
 
     def emit(self, out):

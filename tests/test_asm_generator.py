@@ -57,9 +57,12 @@ def test_kernel_text_invariants(gen, kw, ragged, packed):
     # first step of a tile: 16 MFMAs from the constant 0 (15 in the second copy); a merging segment
     # keeps four accumulators (three of them among MFMAs 1..15)
     assert len(re.findall(r"v_mfma_f32_32x32x2_f32 [^\n]*, 0$", text, re.M)) == (16 + 15) + (12 + 12)
-    # the counted waits rely on exactly 64 stores per epilogue (two epilogues: plain, publishing)
-    assert len(re.findall(r"buffer_store_dword", text)) == 2 * 64
-    assert len(re.findall(r"buffer_store_dword [^\n]* sc0 sc1", text)) == 64
+    # the counted waits rely on exactly 64 stores per epilogue (four epilogues: plain, publishing,
+    # and both again with the partial tile of the next workgroup added, for ranges inside a tile)
+    assert len(re.findall(r"buffer_store_dword", text)) == 4 * 64
+    assert len(re.findall(r"buffer_store_dword [^\n]* sc0 sc1", text)) == 2 * 64
+    # partial tiles are read past the caches: merge_init and the two late merges, 64 loads each
+    assert len(re.findall(r"buffer_load_dword v\d+, [^\n]* sc0 sc1", text)) == 3 * 64
     # s_waitcnt fields: vmcnt has 6 bits, lgkmcnt 4
     assert all(int(n) <= 63 for n in re.findall(r"vmcnt\((\d+)\)", text))
     assert all(int(n) <= 15 for n in re.findall(r"lgkmcnt\((\d+)\)", text))

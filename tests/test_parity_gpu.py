@@ -365,6 +365,39 @@ def test_benchmark_configs_on_hip_kernels(ocn, oracle, torch_gpu, name, N, C, H,
     check_against_oracle(oracle, y, x, w)
 
 
+# layers with tiles for at most half of the compute units: two or four workgroups per tile, the
+# parts of the channel sum handed over through the output tensor in the output transforms
+# (the last flag: whether the tiles are cut - pieces of at least 8 units, an even number of units)
+FEW_TILES = [(32, 512, 7, 7, 512, True), (32, 256, 14, 14, 256, True), (64, 128, 7, 7, 128, True),
+             (32, 64, 8, 8, 64, False), (32, 136, 5, 9, 96, False), (8, 256, 14, 14, 256, True),
+             (20, 200, 6, 6, 250, False), (1, 1024, 7, 7, 1024, True), (32, 384, 9, 5, 320, True)]
+
+
+@pytest.mark.parametrize("N,C,H,W,K,cut", FEW_TILES)
+def test_few_tiles_cut_among_workgroups(ocn, oracle, torch_gpu, N, C, H, W, K, cut):
+    print(f"few tiles N={N} C={C} H={H} W={W} K={K}", flush=True)
+    x, w = make_tensors(ocn, N, C, H, W, K)
+    r = Runner(ocn, torch_gpu, x, w)
+    try:
+        ocn.set_kernel_variant(ocn.KERNEL_ASM)
+        y = r.split()
+        y2 = r.split()
+        ocn.set_balanced_split(False)  # one workgroup per tile: nothing is handed over
+        y1 = r.split()
+    finally:
+        ocn.set_balanced_split(True)
+        ocn.set_kernel_variant(ocn.KERNEL_AUTO)
+    assert not np.isnan(y).any(), "an output element was never written"
+    assert np.array_equal(y, y2)
+    rel64, _, _ = oracle.compare(y, oracle.direct_conv_f64(x, w))
+    assert rel64 <= 1e-5, f"rel-L2 vs fp64 direct {rel64:.3e}"
+    rel1, _, _ = oracle.compare(y, y1)
+    # cut tiles: another association of the channel sum; else the same launch
+    assert (0 < rel1 <= 1e-6) if cut else rel1 == 0, f"rel-L2 vs one workgroup per tile {rel1:.3e}"
+    if H == W:
+        check_against_oracle(oracle, y, x, w)
+
+
 def test_assembly_variant_rejects_launches_it_does_not_take(ocn, torch_gpu):
     # 450 workgroup tiles on 256 compute units need the balanced split, which is switched off
     x, w = make_tensors(ocn, 32, 8, 60, 60, 64)
