@@ -164,7 +164,7 @@ int opencnn_set_kernel_variant(int variant);
  * between two workgroups is merged through the output tensor and two words of library-owned
  * device state per wave.  Results stay independent of timing (two addends commute).  The same
  * hand-over serves layers with tiles for at most half of the compute units (small batches on
- * deep layers, fp32 operands): every tile is cut among two or four workgroups, and the parts of
+ * deep layers): every tile is cut among two or four workgroups, and the parts of
  * its channel sum are passed from workgroup to workgroup in a fixed order.  That
  * state exists once per stream for the first eight streams that launch (calls on different
  * streams may overlap in time); calls on further streams run without the split.  Pass 0 to

@@ -286,7 +286,7 @@ int pieces_per_tile(int nblocks, int chunks, int cus) {
   return pieces;
 }
 
-// cut_tiles: the kernel can merge in its output transform (the fp32 kernels).
+// cut_tiles: whether the caller wants the tiles of a small layer cut.
 int asm_grid(const opencnn::ConvArgs& a, int kw, int chunks, bool cut_tiles, int* grid) {
   *grid = 0;
   if (kw == 1 || (long long)a.nblocks * chunks > kMaxElems) return 0;
@@ -448,9 +448,11 @@ int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* lau
   a.nblocks = (int)nblocks;
   a.colblocks = a.colgroups;
   int grid = 0;
-  // (tiles are not cut: these kernels cannot merge in their output transform)
-  if (int e = asm_grid(a, 4, chunks, false, &grid)) return e;
+  if (int e = asm_grid(a, 4, chunks, true, &grid)) return e;
   if (grid == 0) return 0;
+  // tiles cut among several workgroups (a layer with few tiles): equal pieces, so the weighted
+  // line carries no output transforms
+  const bool cut_tiles = grid > a.nblocks;
   const AsmKernels* ak = nullptr;
   if (int e = asm_kernels(&ak)) return e;
   AsmLaunch l;
@@ -468,7 +470,7 @@ int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* lau
   l.lds_bytes = 2 * 16 * 2 * 4 * 32 * sizeof(unsigned);  // two buffers of V
   l.chunks = chunks;
   l.usw_bytes = usw_bytes;
-  l.epilogue_half_units = kEpilogueHalfUnits;
+  l.epilogue_half_units = cut_tiles ? 0 : kEpilogueHalfUnits;
   l.filters = a.K;
   // How the units are dealt.  While the whole 2-byte transformed filter leaves room in an XCD's
   // 4 MB L2 and the filter blocks are a power of two that divides the grid: one line of units per

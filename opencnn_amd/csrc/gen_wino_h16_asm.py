@@ -121,8 +121,12 @@ class KernelH16(Kernel):
         e(f"s_cmp_eq_u32 {self.sr('Cm')}, 0")
         e(f"s_cselect_b32 {self.sr('N1')}, {self.sr('Chunks')}, {t(0)}")
         e(f"s_cselect_b32 {self.sr('Sfull')}, 0, {t(0)}")
-        for n in ("Cm", "Cp", "Cq"):
-            e(f"s_mov_b32 {self.sr(n)}, 0")
+        # A range shorter than a tile (a layer with few tiles, several workgroups per tile) works
+        # on its own chunks, Cm .. Cm + Nunits - 1, in order: the pieces of a tile must not overlap.
+        e(f"s_cmp_lt_u32 {self.sr('Nunits')}, {self.sr('Chunks')}")
+        e(f"s_cselect_b32 {self.sr('Cm')}, {self.sr('Cm')}, 0")
+        for n in ("Cp", "Cq"):
+            e(f"s_mov_b32 {self.sr(n)}, {self.sr('Cm')}")
 
     def advance_cursor(self, T, C, ahead, hint, on_switch):
         """Cursor (T, C) -> unit G+ahead when there is one: next chunk index modulo Chunks; the
@@ -150,6 +154,9 @@ class KernelH16(Kernel):
         self.e(f"s_branch {back}")
         self.outofline.extend(self.lines)
         self.lines = main
+
+    def late_merge_registers(self):
+        return [self.V["U"] + i for i in range(64)]
 
     def advance_p(self, ahead=3):
         def switch():
@@ -550,8 +557,11 @@ class KernelH16(Kernel):
         seg_loop, done, plain_seg, after_epi, epi = (self.newlabel(x) for x in
                                                      ("seg", "done", "plainseg", "afterepi", "epi"))
         check = [self.newlabel("check0"), self.newlabel("check1")]
+        late_seg, late, late_pub, flag = (self.newlabel(x) for x in ("lateseg", "late", "latepub", "flag"))
         self.stamp()
         self.label(seg_loop)
+        e(f"s_cmp_lt_u32 {self.sr('Nunits')}, {self.sr('Chunks')}")
+        e(f"s_cbranch_scc1 {late_seg}")
         # this segment: the units of tile Tm that belong to this workgroup; SegEnd in units of G.
         # Kind: 1 publish (the range starts inside the tile), 2 merge (it ends inside), 0 whole tile.
         e(f"s_cmp_eq_u32 {self.sr('G')}, 0")
@@ -599,10 +609,13 @@ class KernelH16(Kernel):
         pub = self.newlabel("publish")
         e(f"s_cmp_eq_u32 {self.sr('Kind')}, 1")
         e(f"s_cbranch_scc1 {pub}")
+        e(f"s_cmp_ge_u32 {self.sr('Kind')}, 4")
+        e(f"s_cbranch_scc1 {late}")
         self.epilogue(False)
         e(f"s_branch {after_epi}")
         self.label(pub)
         self.epilogue(True)
+        self.label(flag)
         e("s_waitcnt vmcnt(0)")  # every write-through store acknowledged, then the flag
         self.flag_address(True)
         self.store_flag(self.vr("One"))
@@ -620,6 +633,25 @@ class KernelH16(Kernel):
         e(f"s_branch {seg_loop}")
         self.label(done)
         e("s_endpgm")
+        # A range inside one tile (Kernel.late_merge_loads): its only segment.  Kind 1: the last
+        # piece of the tile, it publishes; 4: the first, it merges and stores the tile; 5: both.
+        self.label(late_seg)
+        e(f"s_cmp_lg_u32 {self.sr('Cm')}, 0")
+        e(f"s_cselect_b32 {self.sr('Kind')}, 1, 0")
+        e(f"s_add_u32 {t(1)}, {self.sr('Cm')}, {self.sr('Nunits')}")
+        e(f"s_or_b32 {t(0)}, {self.sr('Kind')}, 4")
+        e(f"s_cmp_lt_u32 {t(1)}, {self.sr('Chunks')}")
+        e(f"s_cselect_b32 {self.sr('Kind')}, {t(0)}, {self.sr('Kind')}")
+        e(f"s_mov_b32 {self.sr('SegEnd')}, {self.sr('Nunits')}")
+        e(f"s_branch {plain_seg}")
+        self.label(late)
+        e(f"s_cmp_eq_u32 {self.sr('Kind')}, 5")
+        e(f"s_cbranch_scc1 {late_pub}")
+        self.epilogue(False, merge=True)
+        e(f"s_branch {after_epi}")
+        self.label(late_pub)
+        self.epilogue(True, merge=True)
+        e(f"s_branch {flag}")
         self.lines.extend(self.outofline)
 
 
