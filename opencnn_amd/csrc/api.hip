@@ -384,18 +384,27 @@ int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmLaunch& l, hipStream_
 // (spatial tile, batch element) pairs on one line and cut it into column tiles of 32, so only the
 // last column tile has empty columns.  A packed column tile costs 5-8 % more (its lanes' loads
 // straddle two spatial tiles), so: only when an eighth or more of the columns would be empty, and
-// when the unpacked layer (unpacked_tiles workgroup tiles) has more than one round of tiles for
-// the compute units - a layer that fits one round takes one tile's time either way.
+// when fewer tiles make the layer shorter - it has more than one round of workgroup tiles for the
+// compute units, or the packed tiles can be cut into more pieces (pieces_per_tile); otherwise the
+// layer takes one tile's time either way.  cw = column tiles per workgroup tile, kblocks = the
+// filter blocks, chunks = units per tile.
 // Returns whether the shape is packed; *a then holds the packed column tiles.
-int pack_columns(opencnn::ConvArgs* a, long long unpacked_tiles, bool* packed) {
+int pack_columns(opencnn::ConvArgs* a, int cw, int kblocks, int chunks, bool* packed) {
   *packed = false;
   if (a->N % 32 == 0 || a->N * 8 > a->ngroups * 32 * 7) return 0;
   int cus = 0;
   if (int e = compute_units(&cus)) return e;
-  if (unpacked_tiles <= cus) return 0;
   const long long columns = (long long)a->tiles_h * a->tiles_w * a->N;  // below 2^31: it divides the output
+  const long long packed_colgroups = (columns + 31) / 32;
+  const long long unpacked_tiles = ((long long)a->colgroups + cw - 1) / cw * kblocks;
+  const long long packed_tiles = (packed_colgroups + cw - 1) / cw * kblocks;
+  if (unpacked_tiles <= cus) {
+    const bool split = g_balance.load() != 0 && a->sync != nullptr;
+    if (!split || pieces_per_tile((int)packed_tiles, chunks, cus) <= pieces_per_tile((int)unpacked_tiles, chunks, cus))
+      return 0;
+  }
   a->ngroups = 1;
-  a->colgroups = (int)((columns + 31) / 32);
+  a->colgroups = (int)packed_colgroups;
   *packed = true;
   return 0;
 }
@@ -434,7 +443,7 @@ constexpr int kEpilogueHalfUnits = 3;
 int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* launched) {
   *launched = false;
   bool packed = false;
-  if (int e = pack_columns(&a, (long long)a.colgroups * ((a.kgroups + 3) / 4), &packed)) return e;
+  if (int e = pack_columns(&a, 1, (a.kgroups + 3) / 4, (int)(padded_c_h16(a.C) / 16), &packed)) return e;
   // Any shape.  Waves of the last filter block whose 32 filters do not exist help with the input
   // transform, multiply zeros and store nothing.  In the _ragged kernels the last chunk's missing
   // channels read as zeros (descriptor cut at the tensor's end) and meet zero rows of the padded
@@ -595,9 +604,8 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
     // is faster there (measured, K = 32).
     const int kw = a.kgroups == 1 ? 1 : ((a.kgroups + 3) / 4 * 4 <= (a.kgroups + 1) / 2 * 2 ? 4 : 2);
     opencnn::ConvArgs b = a;
-    REQUIRE(tile_with(b, kw));
     bool packed = false;
-    if (int e = pack_columns(&b, b.nblocks, &packed)) return e;
+    if (int e = pack_columns(&b, 4 / kw, (b.kgroups + kw - 1) / kw, (b.C + 7) / 8, &packed)) return e;
     REQUIRE(tile_with(b, kw));
     int grid = 0;
     if (int e = asm_grid(b, kw, (b.C + 7) / 8, true, &grid)) return e;

@@ -397,8 +397,9 @@ def test_few_tiles_cut_among_workgroups(ocn, oracle, torch_gpu, prec, N, C, H, W
     rel64, _, _ = oracle.compare(y, oracle.direct_conv_f64(x, w))
     assert rel64 <= {"f32": 1e-5, "f16": 2e-3, "bf16": 1.5e-2}[prec], f"rel-L2 vs fp64 direct {rel64:.3e}"
     rel1, _, _ = oracle.compare(y, y1)
-    # cut tiles: another association of the channel sum; else the same launch
-    assert (0 < rel1 <= 1e-6) if cut else rel1 == 0, f"rel-L2 vs one workgroup per tile {rel1:.3e}"
+    # cut tiles: another association of the channel sum (fp32 roundings of up to 1024 addends);
+    # else the same launch
+    assert (0 < rel1 <= 3e-6) if cut else rel1 == 0, f"rel-L2 vs one workgroup per tile {rel1:.3e}"
     if H == W and prec == "f32":
         check_against_oracle(oracle, y, x, w)
 
@@ -455,14 +456,16 @@ def test_buffers_need_only_float_alignment(ocn, oracle, torch_gpu, family, prec,
 # batches that are no multiple of 32: the assembly kernels cut their column tiles from the line of
 # all (spatial tile, batch element) pairs, so a column tile holds several tiles or parts of two.
 # The library packs when an eighth of the columns would be empty and the layer has more workgroup
-# tiles than compute units; the last four shapes stay on the unpacked _ragged kernels.
+# tiles than compute units, or when fewer tiles can be cut into more pieces (N = 8 on the deep
+# layer: with fp32 units only); the other three of the last four shapes stay on the unpacked
+# _ragged kernels.
 PACKED_SHAPES = [(1, 8, 64, 64, 64, True), (2, 16, 47, 39, 128, True), (3, 8, 45, 45, 64, True),
                  (5, 24, 33, 37, 100, True), (7, 3, 41, 50, 40, True), (9, 40, 36, 36, 250, True),
                  (12, 20, 40, 30, 160, True), (16, 64, 56, 56, 64, True), (17, 16, 50, 50, 64, True),
                  (20, 8, 36, 44, 128, True), (33, 24, 23, 23, 96, True), (40, 16, 28, 28, 128, True),
                  (48, 32, 40, 40, 64, True), (100, 128, 28, 28, 128, True), (70, 8, 30, 30, 64, True),
                  (1, 16, 112, 112, 64, True),
-                 (1, 64, 14, 14, 64, False), (8, 256, 14, 14, 256, False), (60, 8, 40, 40, 64, False),
+                 (1, 64, 14, 14, 64, False), (8, 256, 14, 14, 256, "f32"), (60, 8, 40, 40, 64, False),
                  (127, 16, 25, 25, 256, False)]
 
 
@@ -472,6 +475,8 @@ def test_batches_on_packed_column_tiles(ocn, oracle, torch_gpu, prec, N, C, H, W
     # the assembly kernels selected explicitly; against the fp64 direct convolution, the HIP C++
     # kernels (which leave the columns of missing batch elements empty) and a second call
     print(f"packed {prec} N={N} C={C} H={H} W={W} K={K}", flush=True)
+    if isinstance(packed, str):
+        packed = packed == prec
     x, w = make_tensors(ocn, N, C, H, W, K)
     r = Runner(ocn, torch_gpu, x, w)
     try:
