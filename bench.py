@@ -160,6 +160,73 @@ def miopen_column(torch, lay, warmup=10, iters=200, settle_ms=150.0):
     return ev[0].elapsed_time(ev[1]) / iters
 
 
+# (C, K, H = W, how many) of the 3x3 stride-1 layers of two networks
+NETWORKS = {
+    "resnet34": [(64, 64, 56, 6), (128, 128, 28, 7), (256, 256, 14, 11), (512, 512, 7, 5)],
+    "vgg16": [(3, 64, 224, 1), (64, 64, 224, 1), (64, 128, 112, 1), (128, 128, 112, 1), (128, 256, 56, 1),
+              (256, 256, 56, 2), (256, 512, 28, 1), (512, 512, 28, 2), (512, 512, 14, 3)],
+}
+NETWORK_BATCHES = (("resnet34", 128), ("resnet34", 32), ("resnet34", 8), ("vgg16", 64), ("vgg16", 16))
+
+
+def network_rows(ocn, torch):
+    """Informational: every 3x3 stride-1 layer of a network timed on its own in the sustained
+    state (this library with fp32 and with fp16 GEMM operands; torch conv2d = MIOpen on fp32 and
+    on half tensors), ms summed with the layer counts.  Never an oracle."""
+    import numpy as np
+
+    def ours(N, C, H, K, prec):
+        x = torch.rand(C, H, H, N, device="cuda") * 2 - 1
+        w = torch.randn(C, 3, 3, K, device="cuda") * float(np.sqrt(2 / (9 * C)))
+        y = torch.empty(K, H, H, N, device="cuda")
+        ws = torch.empty(ocn.workspace_bytes(C, K) // 4, device="cuda")
+        iters = int(max(30, min(1000, 0.15 / (2.0 * N * K * C * H * H * 9 / 200e12))))
+        try:
+            ocn.set_operand_precision(prec)
+            ocn.time_forward(x, w, y, ws, N, C, H, H, K, warmup=3, iters=iters)  # settles the device
+            total, _, _ = ocn.time_forward(x, w, y, ws, N, C, H, H, K, warmup=3, iters=iters)
+        finally:
+            ocn.set_operand_precision(ocn.F32)
+        return total, ocn.last_kernel()
+
+    def miopen(N, C, H, K, dtype):
+        x = (torch.rand(N, C, H, H, device="cuda") * 2 - 1).to(dtype)
+        w = (torch.randn(K, C, 3, 3, device="cuda") * float(np.sqrt(2 / (9 * C)))).to(dtype)
+        torch.backends.cudnn.benchmark = True
+        iters = int(max(30, min(1000, 0.15 / (2.0 * N * K * C * H * H * 9 / 100e12))))
+        for _ in range(10):
+            torch.nn.functional.conv2d(x, w, padding=1)
+        torch.cuda.synchronize()
+        for _ in range(2):  # the first pass settles the device
+            ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+            ev[0].record()
+            for _ in range(iters):
+                torch.nn.functional.conv2d(x, w, padding=1)
+            ev[1].record()
+            torch.cuda.synchronize()
+        return ev[0].elapsed_time(ev[1]) / iters
+
+    rows = []
+    for net, N in NETWORK_BATCHES:
+        row = {"network": net, "N": N, "ms_fp32": 0.0, "ms_fp16_operands": 0.0, "ms_miopen_fp32": 0.0,
+               "ms_miopen_fp16_tensors": 0.0, "layers": []}
+        for C, K, H, count in NETWORKS[net]:
+            a, ka = ours(N, C, H, K, ocn.F32)
+            b, kb = ours(N, C, H, K, ocn.F16)
+            m32, m16 = miopen(N, C, H, K, torch.float32), miopen(N, C, H, K, torch.float16)
+            row["layers"].append({"C": C, "K": K, "H": H, "count": count, "ms_fp32": a, "ms_fp16_operands": b,
+                                  "ms_miopen_fp32": m32, "ms_miopen_fp16_tensors": m16,
+                                  "kernel_fp32": ka, "kernel_fp16_operands": kb})
+            row["ms_fp32"] += a * count
+            row["ms_fp16_operands"] += b * count
+            row["ms_miopen_fp32"] += m32 * count
+            row["ms_miopen_fp16_tensors"] += m16 * count
+            print(f"bench.py --networks: {net} N={N} {C}->{K} {H}x{H}: {a:.4f} / {b:.4f} ms, "
+                  f"MIOpen {m32:.4f} / {m16:.4f} ms", file=sys.stderr, flush=True)  # a long run stays audible
+        rows.append(row)
+    return rows
+
+
 def timeline_summary(ocn, torch, lay, launches=20, operands="f32", settle_ms=150.0):
     """Where a launch of the assembly kernels spends its time: per-workgroup stamps (kernel start,
     end of the prologue, before / after every output transform) of the last of `launches`
@@ -253,6 +320,9 @@ def main():
     ap.add_argument("--shims", action="store_true",
                     help="add the layout shims and the filter transform (HBM-bound kernels) of every "
                          "fp32 layer to the output")
+    ap.add_argument("--networks", action="store_true",
+                    help="add the summed 3x3 layers of ResNet-34 and VGG-16 at several batch sizes, with "
+                         "informational MIOpen columns (takes about a minute)")
     ap.add_argument("--miopen", action="store_true",
                     help="add an informational MIOpen (torch conv2d, fp32) column to the per-layer table")
     args = ap.parse_args()
@@ -374,6 +444,9 @@ def main():
                 out["timeline"].append(timeline_summary(ocn, torch, lay))
             del lay
         out["layers"] = rows
+
+    if args.networks:
+        out["networks"] = network_rows(ocn, torch)
 
     print(json.dumps(out))
 
