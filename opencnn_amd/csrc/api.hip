@@ -268,26 +268,45 @@ int launch_h16(opencnn::ConvArgs a, int precision, hipStream_t st) {
   return launched_hip("wino_h16_fused_lds");
 }
 
-// Grid of the hand-scheduled kernels for this layer, or 0 when they do not take it.  One
-// persistent launch whose workgroups share the (tile, chunk) units evenly; it needs whole filter
-// blocks (kw > 1) and at least one tile per workgroup (a tile then has at most two contributors).
-// A layer with tiles for at most half of the compute units: every tile is cut into `pieces`
-// equal runs of units, one workgroup each.  The last piece publishes its part of the outputs,
-// every other one adds the part published behind it in its output transform and publishes the
-// sum, the first stores the tile: a chain of pieces - 1 hand-overs of about 5 us behind
-// 1 / pieces of the tile's units.  Pieces of at least kMinUnitsPerPiece units.
-constexpr int kMinUnitsPerPiece = 8;
+// A layer with fewer workgroup tiles than compute units would run one tile per workgroup, serially,
+// on a part of the chip.  Instead its units are dealt to more workgroups than it has tiles.  A
+// workgroup whose range ends inside a tile adds, in its output transform, the partial tile that
+// the workgroup behind it published, and publishes the sum if its range also started inside
+// that tile; the workgroup with the tile's first units stores the tile: per tile a chain of
+// hand-overs of about 4 us each, in a fixed order.  Ranges of at least kMinUnitsPerRange units.
+constexpr int kMinUnitsPerRange = 8;
+
+// How a kernel family can cut the tiles of such a layer.
+enum CutTiles {
+  kCutNone,
+  kCutPieces,  // 2 or 4 equal pieces per tile (fp16 / bf16 kernels: a range stays inside one tile)
+  kCutRanges   // equal ranges of the line of all units, one per compute unit (fp32 kernels)
+};
 
 int pieces_per_tile(int nblocks, int chunks, int cus) {
   int pieces = 1;
   while (pieces < 4 && nblocks * pieces * 2 <= cus && nblocks * pieces * 2 <= opencnn::kMaxBalancedBlocks &&
-         chunks % (pieces * 2) == 0 && chunks / (pieces * 2) >= kMinUnitsPerPiece)
+         chunks % (pieces * 2) == 0 && chunks / (pieces * 2) >= kMinUnitsPerRange)
     pieces *= 2;
   return pieces;
 }
 
-// cut_tiles: whether the caller wants the tiles of a small layer cut.
-int asm_grid(const opencnn::ConvArgs& a, int kw, int chunks, bool cut_tiles, int* grid) {
+// Workgroups for nblocks < cus tiles of `chunks` units cut into equal ranges: one per compute
+// unit, fewer when the ranges would get shorter than kMinUnitsPerRange (then a multiple of 8,
+// for the XCD-aware block order); nblocks when that does not cut anything.
+int ranges_for_few_tiles(int nblocks, int chunks, int cus) {
+  const long long total = (long long)nblocks * chunks;
+  long long grid = total / kMinUnitsPerRange;
+  if (grid > cus) grid = cus;
+  if (grid > opencnn::kMaxBalancedBlocks) grid = opencnn::kMaxBalancedBlocks;
+  if (grid >= 8) grid -= grid % 8;
+  return grid > nblocks ? (int)grid : nblocks;
+}
+
+// Grid of the hand-scheduled kernels for this layer, or 0 when they do not take it.  One
+// persistent launch whose workgroups share the (tile, chunk) units evenly; it needs filter blocks
+// of kw > 1 groups.  With at least one tile per workgroup a tile has at most two contributors.
+int asm_grid(const opencnn::ConvArgs& a, int kw, int chunks, CutTiles cut, int* grid) {
   *grid = 0;
   if (kw == 1 || (long long)a.nblocks * chunks > kMaxElems) return 0;
   // per-lane store offsets: four filter rows plus one image row and column, in bytes
@@ -297,7 +316,8 @@ int asm_grid(const opencnn::ConvArgs& a, int kw, int chunks, bool cut_tiles, int
   const bool split = g_balance.load() != 0 && a.sync != nullptr;
   if (a.nblocks < cus) {
     *grid = a.nblocks;  // one tile per workgroup
-    if (cut_tiles && split) *grid = a.nblocks * pieces_per_tile(a.nblocks, chunks, cus);
+    if (split && cut == kCutPieces) *grid = a.nblocks * pieces_per_tile(a.nblocks, chunks, cus);
+    if (split && cut == kCutRanges) *grid = ranges_for_few_tiles(a.nblocks, chunks, cus);
   } else if (cus % 8 == 0 && cus <= opencnn::kMaxBalancedBlocks && (a.nblocks % cus == 0 || split)) {
     *grid = cus;
   }
@@ -389,7 +409,7 @@ int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmLaunch& l, hipStream_
 // layer takes one tile's time either way.  cw = column tiles per workgroup tile, kblocks = the
 // filter blocks, chunks = units per tile.
 // Returns whether the shape is packed; *a then holds the packed column tiles.
-int pack_columns(opencnn::ConvArgs* a, int cw, int kblocks, int chunks, bool* packed) {
+int pack_columns(opencnn::ConvArgs* a, int cw, int kblocks, int chunks, CutTiles cut, bool* packed) {
   *packed = false;
   if (a->N % 32 == 0 || a->N * 8 > a->ngroups * 32 * 7) return 0;
   int cus = 0;
@@ -400,8 +420,12 @@ int pack_columns(opencnn::ConvArgs* a, int cw, int kblocks, int chunks, bool* pa
   const long long packed_tiles = (packed_colgroups + cw - 1) / cw * kblocks;
   if (unpacked_tiles <= cus) {
     const bool split = g_balance.load() != 0 && a->sync != nullptr;
-    if (!split || pieces_per_tile((int)packed_tiles, chunks, cus) <= pieces_per_tile((int)unpacked_tiles, chunks, cus))
+    if (!split) return 0;
+    // (cut into ranges, the layer's time follows its number of units: fewer tiles, fewer units)
+    if (cut == kCutPieces &&
+        pieces_per_tile((int)packed_tiles, chunks, cus) <= pieces_per_tile((int)unpacked_tiles, chunks, cus))
       return 0;
+    if (cut == kCutRanges && ranges_for_few_tiles((int)unpacked_tiles, chunks, cus) == unpacked_tiles) return 0;
   }
   a->ngroups = 1;
   a->colgroups = (int)packed_colgroups;
@@ -443,7 +467,7 @@ constexpr int kEpilogueHalfUnits = 3;
 int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* launched) {
   *launched = false;
   bool packed = false;
-  if (int e = pack_columns(&a, 1, (a.kgroups + 3) / 4, (int)(padded_c_h16(a.C) / 16), &packed)) return e;
+  if (int e = pack_columns(&a, 1, (a.kgroups + 3) / 4, (int)(padded_c_h16(a.C) / 16), kCutPieces, &packed)) return e;
   // Any shape.  Waves of the last filter block whose 32 filters do not exist help with the input
   // transform, multiply zeros and store nothing.  In the _ragged kernels the last chunk's missing
   // channels read as zeros (descriptor cut at the tensor's end) and meet zero rows of the padded
@@ -457,7 +481,7 @@ int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* lau
   a.nblocks = (int)nblocks;
   a.colblocks = a.colgroups;
   int grid = 0;
-  if (int e = asm_grid(a, 4, chunks, true, &grid)) return e;
+  if (int e = asm_grid(a, 4, chunks, kCutPieces, &grid)) return e;
   if (grid == 0) return 0;
   // tiles cut among several workgroups (a layer with few tiles): equal pieces, so the weighted
   // line carries no output transforms
@@ -605,10 +629,10 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
     const int kw = a.kgroups == 1 ? 1 : ((a.kgroups + 3) / 4 * 4 <= (a.kgroups + 1) / 2 * 2 ? 4 : 2);
     opencnn::ConvArgs b = a;
     bool packed = false;
-    if (int e = pack_columns(&b, 4 / kw, (b.kgroups + kw - 1) / kw, (b.C + 7) / 8, &packed)) return e;
+    if (int e = pack_columns(&b, 4 / kw, (b.kgroups + kw - 1) / kw, (b.C + 7) / 8, kCutRanges, &packed)) return e;
     REQUIRE(tile_with(b, kw));
     int grid = 0;
-    if (int e = asm_grid(b, kw, (b.C + 7) / 8, true, &grid)) return e;
+    if (int e = asm_grid(b, kw, (b.C + 7) / 8, kCutRanges, &grid)) return e;
     if (grid > 0)
       return launch_asm(b, kw, grid, ragged || b.kgroups % kw != 0, packed, lds_bytes(kw), st);
     REQUIRE(variant != OPENCNN_KERNEL_ASM);

@@ -365,20 +365,25 @@ def test_benchmark_configs_on_hip_kernels(ocn, oracle, torch_gpu, name, N, C, H,
     check_against_oracle(oracle, y, x, w)
 
 
-# layers with tiles for at most half of the compute units: two or four workgroups per tile, the
-# parts of the channel sum handed over through the output tensor in the output transforms
-# (the last flag: whether the tiles are cut - pieces of at least 8 units, an even number of units)
-FEW_TILES = [(32, 512, 7, 7, 512, True), (32, 256, 14, 14, 256, True), (64, 128, 7, 7, 128, True),
-             (32, 64, 8, 8, 64, False), (32, 136, 5, 9, 96, False), (8, 256, 14, 14, 256, True),
-             (20, 200, 6, 6, 250, False), (1, 1024, 7, 7, 1024, True), (32, 384, 9, 5, 320, True)]
+# layers with fewer tiles than compute units: the units are dealt to more workgroups than tiles,
+# the parts of a tile's channel sum handed over through the output tensor in the output
+# transforms.  fp32 kernels: equal ranges of at least 8 units over the line of all units (a range
+# may cross a tile boundary); fp16 / bf16 kernels: 2 or 4 equal pieces per tile of at least 8 of
+# their 16-channel units.  The flags: whether the fp32 / the fp16 and bf16 kernels cut the layer.
+FEW_TILES = [(32, 512, 7, 7, 512, True, True), (32, 256, 14, 14, 256, True, True),
+             (64, 128, 7, 7, 128, True, False), (32, 64, 8, 8, 64, False, False),
+             (32, 136, 5, 9, 96, True, False), (8, 256, 14, 14, 256, True, True),
+             (20, 200, 6, 6, 250, True, False), (1, 1024, 7, 7, 1024, True, True),
+             (32, 384, 9, 5, 320, True, True), (96, 512, 7, 7, 512, True, False),
+             (64, 256, 14, 14, 256, True, False), (32, 72, 10, 10, 128, False, False),
+             (32, 160, 10, 10, 128, True, False)]
 
 
 @pytest.mark.parametrize("prec", ["f32", "f16", "bf16"])
-@pytest.mark.parametrize("N,C,H,W,K,cut", FEW_TILES)
-def test_few_tiles_cut_among_workgroups(ocn, oracle, torch_gpu, prec, N, C, H, W, K, cut):
+@pytest.mark.parametrize("N,C,H,W,K,cut_f32,cut_h16", FEW_TILES)
+def test_few_tiles_cut_among_workgroups(ocn, oracle, torch_gpu, prec, N, C, H, W, K, cut_f32, cut_h16):
     print(f"few tiles {prec} N={N} C={C} H={H} W={W} K={K}", flush=True)
-    if prec != "f32":  # units of 16 channels: pieces of at least 8 of them, an even number
-        cut = cut and C % 32 == 0 and C >= 256
+    cut = cut_f32 if prec == "f32" else cut_h16
     x, w = make_tensors(ocn, N, C, H, W, K)
     r = Runner(ocn, torch_gpu, x, w)
     try:
