@@ -296,7 +296,11 @@ int pieces_per_tile(int nblocks, int chunks, int cus) {
 // for the XCD-aware block order); nblocks when that does not cut anything.
 int ranges_for_few_tiles(int nblocks, int chunks, int cus) {
   const long long total = (long long)nblocks * chunks;
-  long long grid = total / kMinUnitsPerRange;
+  // A tile of `chunks` units cut into p ranges takes chunks / p units and p - 1 hand-overs of
+  // about two units each: shortest near p = sqrt(chunks / 2), i.e. ranges of sqrt(2 * chunks) units.
+  int min_units = kMinUnitsPerRange;
+  while (min_units * min_units < 2 * chunks) ++min_units;
+  long long grid = total / min_units;
   if (grid > cus) grid = cus;
   if (grid > opencnn::kMaxBalancedBlocks) grid = opencnn::kMaxBalancedBlocks;
   if (grid >= 8) grid -= grid % 8;
