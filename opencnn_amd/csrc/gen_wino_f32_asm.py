@@ -657,25 +657,43 @@ class Kernel:
         if self.ragged_k:
             self.row_limit(r + 1)
 
+    def output_transform_row(self, r, o):
+        """Accumulator row r of all 16 positions -> its four outputs in o(0..3)
+        (Y = A^T M A, order of src/store_and_transform_output_optSTS64.cuh:29-51)."""
+        m = lambda i: self.vr("T", i)
+        w = lambda i: self.vr("TO", i)          # a_j: 0-3, b_j: 4-7
+        for j in range(4):
+            self.e(f"v_add_f32 {w(j)}, {m(j)}, {m(4 + j)}")
+            self.e(f"v_sub_f32 {w(4 + j)}, {m(4 + j)}, {m(8 + j)}")
+        for j in range(4):
+            self.e(f"v_add_f32 {w(j)}, {w(j)}, {m(8 + j)}")
+            self.e(f"v_sub_f32 {w(4 + j)}, {w(4 + j)}, {m(12 + j)}")
+        self.e(f"v_add_f32 {o(0)}, {w(0)}, {w(1)}")
+        self.e(f"v_sub_f32 {o(1)}, {w(1)}, {w(2)}")
+        self.e(f"v_add_f32 {o(2)}, {w(4)}, {w(5)}")
+        self.e(f"v_sub_f32 {o(3)}, {w(5)}, {w(6)}")
+        self.e(f"v_add_f32 {o(0)}, {o(0)}, {w(2)}")
+        self.e(f"v_sub_f32 {o(1)}, {o(1)}, {w(3)}")
+        self.e(f"v_add_f32 {o(2)}, {o(2)}, {w(6)}")
+        self.e(f"v_sub_f32 {o(3)}, {o(3)}, {w(7)}")
+
     def epilogue(self, through, merge=False):
-        """Y = A^T M A per accumulator element (order of src/store_and_transform_output_optSTS64.cuh:29-51)
-        and the 64 stores of the tile; `through` = write past the caches (a partial tile that a
-        workgroup on another XCD will read).  `merge`: the partial tile that the next workgroup
-        published is added to the outputs here (late_merge)."""
+        """The output transform per accumulator element and the 64 stores of the tile; `through` =
+        write past the caches (a partial tile that a workgroup on another XCD will read).
+        `merge`: the partial tile that the next workgroup published is added (late_merge)."""
         # final outputs are written once and never read again by this kernel: non-temporal, so that
         # they do not push the input patches that neighbouring tiles share out of L2
         pol = " sc0 sc1" if through else " nt"
         ry = self.S["RsrcY"]
+        m = lambda i: self.vr("T", i)
         if merge:
-            land = self.late_merge_loads()
+            return self.late_merge(pol)
         self.row_start()
         # the last MFMAs must have written the accumulators before they are read
         self.e("s_nop 15")
         self.e("s_nop 15")
-        m = lambda i: self.vr("T", i)
         pending = []
         for r in range(16):
-            w = lambda i: self.vr("TO", i)          # a_j: 0-3, b_j: 4-7
             o = lambda q: self.vr("TO", 8 + 4 * (r & 1) + q)  # outputs alternate between two sets
             for p in range(16):
                 self.e(f"v_accvgpr_read_b32 {m(p)}, {a(16 * p + r)}")
@@ -683,30 +701,47 @@ class Kernel:
                 for st in pending:
                     self.e(st)
                 self.row_advance(r - 1)
-            for j in range(4):
-                self.e(f"v_add_f32 {w(j)}, {m(j)}, {m(4 + j)}")
-                self.e(f"v_sub_f32 {w(4 + j)}, {m(4 + j)}, {m(8 + j)}")
-            for j in range(4):
-                self.e(f"v_add_f32 {w(j)}, {w(j)}, {m(8 + j)}")
-                self.e(f"v_sub_f32 {w(4 + j)}, {w(4 + j)}, {m(12 + j)}")
-            self.e(f"v_add_f32 {o(0)}, {w(0)}, {w(1)}")
-            self.e(f"v_sub_f32 {o(1)}, {w(1)}, {w(2)}")
-            self.e(f"v_add_f32 {o(2)}, {w(4)}, {w(5)}")
-            self.e(f"v_sub_f32 {o(3)}, {w(5)}, {w(6)}")
-            self.e(f"v_add_f32 {o(0)}, {o(0)}, {w(2)}")
-            self.e(f"v_sub_f32 {o(1)}, {o(1)}, {w(3)}")
-            self.e(f"v_add_f32 {o(2)}, {o(2)}, {w(6)}")
-            self.e(f"v_sub_f32 {o(3)}, {o(3)}, {w(7)}")
-            if merge:
-                if r == 0:
-                    self.e("s_waitcnt vmcnt(0)")  # the partial tile has landed (no store is out yet)
-                    self.store_flag(self.vr("Zero"))  # hand the flag back for the next launch
-                for q in range(4):
-                    self.e(f"v_add_f32 {o(q)}, {o(q)}, {v(land[r * 4 + q])}")
+            self.output_transform_row(r, o)
             pending = [f"buffer_store_dword {o(q)}, {self.vr('Eff', q)}, {s(ry, 4)}, 0 offen{pol}" for q in range(4)]
             if r == 15:
                 for st in pending:
                     self.e(st)
+
+    def late_merge(self, pol):
+        """The output transform of a range that ends inside a tile of a layer with fewer tiles than
+        compute units.  Every workgroup of such a tile finishes its units at about the same time,
+        so the partial tile of the workgroup behind this one cannot be in the accumulators before
+        the first unit as in merge_init.  All 64 outputs are computed first, into registers;
+        then: wait for the flag, read the partial tile past the caches, add, store.  This is the
+        last thing the workgroup does, so the pipeline's registers are free - once its last
+        prefetches, which nothing waits for any more, have landed."""
+        ry = self.S["RsrcY"]
+        m = lambda i: self.vr("T", i)
+        out, land = self.late_output_registers(), self.late_merge_registers()
+        assert len(set(out + land)) == 128
+        self.comment("---- late merge: outputs first, then the partial tile of the workgroup behind")
+        self.e("s_waitcnt vmcnt(0) lgkmcnt(0)")
+        self.e("s_nop 15")
+        self.e("s_nop 15")
+        for r in range(16):
+            for p in range(16):
+                self.e(f"v_accvgpr_read_b32 {m(p)}, {a(16 * p + r)}")
+            self.output_transform_row(r, lambda q: v(out[r * 4 + q]))
+        self.wait_flag()
+        self.row_start()
+        for r in range(16):
+            for q in range(4):
+                self.e(f"buffer_load_dword {v(land[r * 4 + q])}, {self.vr('Eff', q)}, {s(ry, 4)}, 0 offen sc0 sc1")
+            self.row_advance(r)
+        self.e("s_waitcnt vmcnt(0)")
+        self.store_flag(self.vr("Zero"))  # hand the flag back for the next launch
+        self.row_start()
+        for r in range(16):
+            for q in range(4):
+                self.e(f"v_add_f32 {v(out[r * 4 + q])}, {v(out[r * 4 + q])}, {v(land[r * 4 + q])}")
+            for q in range(4):
+                self.e(f"buffer_store_dword {v(out[r * 4 + q])}, {self.vr('Eff', q)}, {s(ry, 4)}, 0 offen{pol}")
+            self.row_advance(r)
 
     def flag_address(self, previous):
         """Fl = &flags[((L - previous) * 4 + wave) * 2 + 1]."""
@@ -746,26 +781,13 @@ class Kernel:
         self.label(got)
 
     def late_merge_registers(self):
-        """64 registers for a partial tile that is added in the output transform.  That transform is
-        the last thing its workgroup does, so the filter registers are dead; a prefetch into them
-        that is still in flight lands before the partial tile (loads return in order)."""
+        """64 registers for the partial tile of a late merge: the filter operands."""
         return [self.V["U0"] + i for i in range(32)] + [self.V["U1"] + i for i in range(32)]
 
-    def late_merge_loads(self):
-        """A range that lies inside one tile (a layer with few tiles, cut among several
-        workgroups): every workgroup of the tile finishes its units at the same time, so the
-        published part of the tile cannot be in the accumulators before the first unit as in
-        merge_init.  Wait for it here and add it to the outputs (epilogue)."""
-        land = self.late_merge_registers()
-        ry = self.S["RsrcY"]
-        self.comment("---- late merge: the partial tile is added in the output transform")
-        self.wait_flag()
-        self.row_start()
-        for r in range(16):
-            for q in range(4):
-                self.e(f"buffer_load_dword {v(land[r * 4 + q])}, {self.vr('Eff', q)}, {s(ry, 4)}, 0 offen sc0 sc1")
-            self.row_advance(r)
-        return land
+    def late_output_registers(self):
+        """64 registers for the outputs of a late merge: patches and B operands."""
+        names = ["D0", "D1" if self.SPW == 2 else "MPX", "VA", "VB"]
+        return [self.V[n] + i for n in names for i in range(16)]
 
     def merge_init(self):
         """Last segment of a workgroup that ends inside a tile: the first part of that tile was

@@ -158,6 +158,9 @@ class KernelH16(Kernel):
     def late_merge_registers(self):
         return [self.V["U"] + i for i in range(64)]
 
+    def late_output_registers(self):
+        return [self.V[n] + i for n in ("DA0", "DB0", "DA1", "DB1") for i in range(16)]
+
     def advance_p(self, ahead=3):
         def switch():
             self.decode(self.sr("Tp"))
