@@ -866,10 +866,12 @@ def test_random_shapes_on_every_kernel_family(ocn, oracle, torch_gpu, prec, seed
         assert rel64 <= bound, f"rel-L2 vs fp64 direct {rel64:.3e}"
 
 
-@pytest.mark.parametrize("N,C,H,K", [(32, 8, 8, 64), (64, 16, 40, 128)])
+@pytest.mark.parametrize("N,C,H,K", [(32, 8, 8, 64), (64, 16, 40, 128), (32, 256, 7, 256), (8, 128, 28, 128)])
 def test_call_replays_from_a_captured_graph(ocn, oracle, torch_gpu, N, C, H, K):
     # The drop-in call only launches kernels (no allocation, no memset, its device state resets
-    # itself), so it can be captured; the second shape has tiles cut between workgroups.  Replays
+    # itself), so it can be captured; the second shape has tiles cut between workgroups, the third
+    # has fewer tiles than compute units (hand-overs in the output transforms), the fourth packed
+    # column tiles on top of that.  Replays
     # with new inputs, eager launches and synchronisations in between, each checked.
     print(f"graph N={N} C={C} H={H} K={K}", flush=True)
     torch = torch_gpu
