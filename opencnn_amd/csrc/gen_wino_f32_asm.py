@@ -1030,8 +1030,7 @@ class Kernel:
         self.label(flag)
         e("s_waitcnt vmcnt(0)")  # every write-through store acknowledged, then the flag
         self.flag_address(True)
-        self.store_flag(self.vr("One"))
-        e("s_waitcnt vmcnt(0)")
+        self.store_flag(self.vr("One"))  # nothing waits for it: the data it announces is acknowledged
         self.label(after_epi)
         self.stamp()
         e(f"s_cmp_lt_u32 {self.sr('G')}, {self.sr('Nunits')}")
