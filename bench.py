@@ -394,6 +394,9 @@ def main():
             "ms_per_launch": ms_main,
             "hbm_min_bytes": bmin,
             "hbm_gbs_at_min_bytes": bmin / (ms_step * 1e-3) / 1e9,
+            "hbm_frac_of_peak_at_min_bytes": bmin / (ms_step * 1e-3) / 1e9 / PEAK_HBM_GBS,
+            # measured traffic of the fused kernel (rocprof counters) over its measured duration
+            "hbm_frac_of_peak_measured_traffic": (traffic / (ms_main * 1e-3) / 1e9 / PEAK_HBM_GBS) if traffic else None,
             "fx_ms_per_launch": ms_fx,
         },
     }
@@ -437,6 +440,7 @@ def main():
                     "mfma_tflops": m / (mn * 1e-3) / 1e12,
                     "mfma_frac_of_peak": m / (mn * 1e-3) / 1e12 / peak,
                     "hbm_gbs_at_min_bytes": b / (tot * 1e-3) / 1e9,
+                    "hbm_frac_of_peak_at_min_bytes": b / (tot * 1e-3) / 1e9 / PEAK_HBM_GBS,
                 })
             if args.shims and not name.startswith("reduced"):
                 out.setdefault("shims", []).extend(shim_rows(ocn, torch, lay))
