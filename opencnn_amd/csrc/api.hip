@@ -350,6 +350,9 @@ struct AsmLaunch {
   // pairs; the magic number of the image groups then divides by the batch size.
   bool packed = false;
   int epilogue_half_units = -1;
+  // fp16 / bf16 kernels: ranges shorter than a tile, walked in the natural chunk order (flagged in
+  // bit 6 of the units' magic shift, which the kernel's 64-bit shifts ignore)
+  bool natural_order = false;
 };
 
 int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmLaunch& l, hipStream_t st) {
@@ -391,6 +394,7 @@ int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmLaunch& l, hipStream_
   ka.grid_per_xcd = grid % 8 == 0 ? grid / 8 : 0;  // 0: no XCD-aware block order
   ka.timeline = (size_t)grid * 64 * sizeof(long long) <= g_timeline_bytes.load() ? g_timeline.load() : nullptr;
   magic_divisor(chunk_divisor, &ka.m_chunks, &ka.s_chunks);
+  if (l.natural_order) ka.s_chunks |= 64;
   magic_divisor((uint32_t)l.tile_split, &ka.m_colblocks, &ka.s_colblocks);
   if (l.lockstep_log2 >= 0) ka.s_colblocks = (uint32_t)l.lockstep_log2;
   magic_divisor((uint32_t)(l.packed ? a.N : a.ngroups), &ka.m_ngroups, &ka.s_ngroups);
@@ -487,8 +491,11 @@ int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* lau
   int grid = 0;
   if (int e = asm_grid(a, 4, chunks, kCutPieces, &grid)) return e;
   if (grid == 0) return 0;
-  // tiles cut among several workgroups (a layer with few tiles): equal pieces, so the weighted
-  // line carries no output transforms
+  // Tiles cut among several workgroups (a layer with fewer tiles than compute units): equal pieces,
+  // so the weighted line carries no output transforms, and the kernel walks the chunks of a
+  // range in their natural order.  (Equal ranges over all compute units as for fp32 were slower
+  // here: these kernels' units are short, and a range that crosses a tile boundary pays two
+  // output transforms and two hand-overs.)
   const bool cut_tiles = grid > a.nblocks;
   const AsmKernels* ak = nullptr;
   if (int e = asm_kernels(&ak)) return e;
@@ -508,6 +515,7 @@ int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* lau
   l.chunks = chunks;
   l.usw_bytes = usw_bytes;
   l.epilogue_half_units = cut_tiles ? 0 : kEpilogueHalfUnits;
+  l.natural_order = cut_tiles;
   l.filters = a.K;
   // How the units are dealt.  While the whole 2-byte transformed filter leaves room in an XCD's
   // 4 MB L2 and the filter blocks are a power of two that divides the grid: one line of units per

@@ -121,10 +121,14 @@ class KernelH16(Kernel):
         e(f"s_cmp_eq_u32 {self.sr('Cm')}, 0")
         e(f"s_cselect_b32 {self.sr('N1')}, {self.sr('Chunks')}, {t(0)}")
         e(f"s_cselect_b32 {self.sr('Sfull')}, 0, {t(0)}")
-        # A range shorter than a tile (a layer with few tiles, several workgroups per tile) works
-        # on its own chunks, Cm .. Cm + Nunits - 1, in order: the pieces of a tile must not overlap.
-        e(f"s_cmp_lt_u32 {self.sr('Nunits')}, {self.sr('Chunks')}")
+        # A layer with fewer tiles than compute units (the host sets bit 6 of the magic shift Sch,
+        # which 64-bit shifts ignore): the ranges are shorter than a tile and a tile may have
+        # three or more contributors, so every range works on its own chunks in the natural
+        # order - from Cm to the end of its first tile, then from chunk 0 of the next.
+        e(f"s_bitcmp1_b32 {self.sr('Sch')}, 6")
         e(f"s_cselect_b32 {self.sr('Cm')}, {self.sr('Cm')}, 0")
+        e(f"s_cselect_b32 {self.sr('Sfull')}, 0, {self.sr('Sfull')}")
+        e(f"s_cselect_b32 {self.sr('Nlast')}, {self.sr('Chunks')}, {self.sr('Nlast')}")
         for n in ("Cp", "Cq"):
             e(f"s_mov_b32 {self.sr(n)}, {self.sr('Cm')}")
 
@@ -563,7 +567,7 @@ class KernelH16(Kernel):
         late_seg, late, late_pub, flag = (self.newlabel(x) for x in ("lateseg", "late", "latepub", "flag"))
         self.stamp()
         self.label(seg_loop)
-        e(f"s_cmp_lt_u32 {self.sr('Nunits')}, {self.sr('Chunks')}")
+        e(f"s_bitcmp1_b32 {self.sr('Sch')}, 6")
         e(f"s_cbranch_scc1 {late_seg}")
         # this segment: the units of tile Tm that belong to this workgroup; SegEnd in units of G.
         # Kind: 1 publish (the range starts inside the tile), 2 merge (it ends inside), 0 whole tile.
@@ -635,16 +639,21 @@ class KernelH16(Kernel):
         e(f"s_branch {seg_loop}")
         self.label(done)
         e("s_endpgm")
-        # A range inside one tile (Kernel.late_merge_loads): its only segment.  Kind 1: the last
-        # piece of the tile, it publishes; 4: the first, it merges and stores the tile; 5: both.
+        # A segment of a range in the natural chunk order (a layer with fewer tiles than compute
+        # units, Kernel.late_merge): chunks Cm .. of tile Tm, up to the tile's or the range's end.
+        # Kind 1: it starts inside the tile and reaches its end: it publishes; 4: it starts with
+        # the tile and ends inside: it merges and stores the tile; 5: both; 0: a whole tile.
         self.label(late_seg)
+        e(f"s_sub_u32 {t(0)}, {self.sr('Chunks')}, {self.sr('Cm')}")
+        e(f"s_sub_u32 {t(1)}, {self.sr('Nunits')}, {self.sr('G')}")
+        e(f"s_min_u32 {t(0)}, {t(0)}, {t(1)}")
+        e(f"s_add_u32 {self.sr('SegEnd')}, {self.sr('G')}, {t(0)}")
         e(f"s_cmp_lg_u32 {self.sr('Cm')}, 0")
         e(f"s_cselect_b32 {self.sr('Kind')}, 1, 0")
-        e(f"s_add_u32 {t(1)}, {self.sr('Cm')}, {self.sr('Nunits')}")
+        e(f"s_add_u32 {t(1)}, {self.sr('Cm')}, {t(0)}")
         e(f"s_or_b32 {t(0)}, {self.sr('Kind')}, 4")
         e(f"s_cmp_lt_u32 {t(1)}, {self.sr('Chunks')}")
         e(f"s_cselect_b32 {self.sr('Kind')}, {t(0)}, {self.sr('Kind')}")
-        e(f"s_mov_b32 {self.sr('SegEnd')}, {self.sr('Nunits')}")
         e(f"s_branch {plain_seg}")
         self.label(late)
         e(f"s_cmp_eq_u32 {self.sr('Kind')}, 5")
