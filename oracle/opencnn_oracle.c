@@ -44,6 +44,13 @@
  *                            fp32 accumulate; no counterpart in the reference
  *                            (it is fp32 only), checked against the fp64 direct
  *                            convolution with the looser bound stated in the tests.
+ *   oracle_round_operand     the RNE roundings of that variant.  Pinned against numpy's
+ *                            float16 cast, torch's CPU bfloat16 / float16 casts and
+ *                            round-to-nearest-even written from its definition in exact
+ *                            rationals (ties of both parities, carries, subnormals,
+ *                            overflow, signed zeros).
+ *   oracle_compare_*         the error metric (relative L2, max |diff|, max |want|).
+ *                            Pinned against numpy norms; NaN / Inf poison both figures.
  *
  * Layouts (all row-major, last index fastest):
  *   x   CHWN  [C][H][W][N]   src/openCNN_winograd.cu:149-150,230

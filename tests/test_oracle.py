@@ -158,17 +158,115 @@ def test_winograd_linearity(oracle):
     assert np.array_equal(lhs, rhs)
 
 
-def test_rounding_helpers(oracle):
-    # fp16 / bf16 round-to-nearest-even against numpy's float16 and a manual bf16
+def _rounding_cases():
+    """float32 values that separate a correct round-to-nearest-even from its plausible mistakes:
+    random values, exact ties (both neighbours' parities), one ulp either side of a tie, carries
+    into the exponent, subnormals of the narrow format, overflow to infinity, signed zeros,
+    infinities."""
     rng = np.random.default_rng(9)
-    vals = np.concatenate([rng.uniform(-4, 4, 200), rng.uniform(-1e-6, 1e-6, 50),
-                           [0.0, 1.0, 65504.0, 70000.0, 2.0 ** -24, 2.0 ** -25, 1.0009765625]])
-    for v in vals.astype(np.float32):
-        with np.errstate(over="ignore"):
-            assert oracle.round_operand(v, 1) == float(np.float32(np.float16(v)))
-        u = np.float32(v).view(np.uint32)
-        bf = np.uint32((int(u) + 0x7FFF + ((int(u) >> 16) & 1)) & 0xFFFF0000).view(np.float32)
-        assert oracle.round_operand(v, 2) == float(bf)
+    bits = rng.integers(0, 1 << 32, 20000, dtype=np.uint64).astype(np.uint32)
+    bits = bits[(bits & 0x7F800000) != 0x7F800000]                       # finite
+    ties16 = (bits[:5000] & np.uint32(0xFFFF0000)) | np.uint32(0x8000)   # bf16 ties
+    ties13 = (rng.integers(0x38800000, 0x47000000, 5000).astype(np.uint32) & np.uint32(0xFFFFE000)) | np.uint32(0x1000)
+    near = np.concatenate([ties16 + np.uint32(1), ties16 - np.uint32(1), ties13 + np.uint32(1), ties13 - np.uint32(1)])
+    carries = np.array([0x3F7FFFFF, 0x3F7F8000, 0x3F7F7FFF, 0x477FEFFF, 0x477FF000, 0x477FE000, 0x7F7FFFFF,
+                        0x7F7F8000, 0x7F7F7FFF, 0x00000001, 0x00008000, 0x00018000, 0x80000000, 0x00000000,
+                        0x7F800000, 0xFF800000], dtype=np.uint32)
+    sub16 = np.float32(2.0 ** -24) * np.array([0.25, 0.5, 0.75, 1.0, 1.5, 2.5, 3.5, 1023.5, 1024.5], dtype=np.float32)
+    small = rng.uniform(-1e-4, 1e-4, 3000).astype(np.float32)             # fp16 subnormal range and around it
+    typical = rng.uniform(-4, 4, 3000).astype(np.float32)
+    big = np.array([65504.0, 65519.996, 65520.0, 65536.0, 70000.0, -65520.0, -65519.996], dtype=np.float32)
+    v = np.concatenate([bits.view(np.float32), ties16.view(np.float32), ties13.view(np.float32),
+                        near.view(np.float32), carries.view(np.float32), sub16, -sub16, small, typical, big])
+    return v[~np.isnan(v)]
+
+
+def _nearest_even_on_grid(v: float, mant_bits: int, emin: int, emax: int) -> float:
+    """Round-to-nearest-even of a finite double onto the binary format with `mant_bits` stored
+    mantissa bits, normal exponents emin..emax and gradual underflow, from the definition (no bit
+    tricks): the two neighbouring grid points in exact arithmetic, the nearer one, the one with
+    the even significand on a tie; beyond the largest finite value plus half a step: infinity."""
+    from fractions import Fraction
+    import math
+    if v == 0.0 or math.isinf(v):
+        return v
+    a = Fraction(abs(v))
+    e = max(math.floor(math.log2(abs(v))), emin)
+    while Fraction(2) ** (e + 1) <= a:
+        e += 1
+    while e > emin and Fraction(2) ** e > a:
+        e -= 1
+    step = Fraction(2) ** (e - mant_bits)
+    q, r = divmod(a, step)
+    if 2 * r > step or (2 * r == step and q % 2 == 1):
+        q += 1
+    out = q * step
+    largest = (Fraction(2) - Fraction(2) ** -mant_bits) * Fraction(2) ** emax
+    if out > largest:
+        return math.copysign(math.inf, v)
+    return math.copysign(float(out), v)
+
+
+def test_rounding_to_fp16_and_bf16_against_library_casts(oracle):
+    # the oracle's RNE helpers against two independent implementations: numpy's float16 cast and
+    # torch's CPU bfloat16 / float16 casts
+    import torch
+    v = _rounding_cases()
+    got16 = np.array([oracle.round_operand(x, 1) for x in v], dtype=np.float32)
+    got_bf = np.array([oracle.round_operand(x, 2) for x in v], dtype=np.float32)
+    with np.errstate(over="ignore"):
+        want16_np = v.astype(np.float16).astype(np.float32)
+    t = torch.from_numpy(v.copy())
+    want16_t = t.to(torch.float16).to(torch.float32).numpy()
+    want_bf = t.to(torch.bfloat16).to(torch.float32).numpy()
+    assert np.array_equal(got16.view(np.uint32), want16_np.view(np.uint32))
+    assert np.array_equal(got16.view(np.uint32), want16_t.view(np.uint32))
+    assert np.array_equal(got_bf.view(np.uint32), want_bf.view(np.uint32))
+    # the cases do exercise what they are for
+    assert np.isinf(got16[np.isfinite(v)]).any() and (got_bf != v).any() and (got16 != v).any()
+
+
+def test_rounding_to_fp16_and_bf16_from_the_definition(oracle):
+    # ... and against round-to-nearest-even written from its definition in exact rationals
+    # (binary16: 10 mantissa bits, exponents -14..15; bfloat16: 7 bits, -126..127)
+    v = _rounding_cases()
+    rng = np.random.default_rng(10)
+    sample = np.concatenate([v[rng.integers(0, v.size, 1500)], v[-40:]])
+    for x in sample:
+        x = float(x)
+        assert oracle.round_operand(x, 1) == _nearest_even_on_grid(x, 10, -14, 15), x
+        want = _nearest_even_on_grid(x, 7, -126, 127)
+        got = oracle.round_operand(x, 2)
+        assert got == want and np.signbit(got) == np.signbit(want), x
+    assert oracle.round_operand(1.5, 0) == 1.5 and oracle.round_operand(1.0 + 2.0 ** -20, 0) == 1.0 + 2.0 ** -20
+
+
+def test_compare_metric_against_numpy(oracle):
+    # oracle.compare is the metric every parity verdict goes through: (rel_l2, max_abs, max_ref)
+    rng = np.random.default_rng(11)
+    for want_dtype in (np.float32, np.float64):
+        want = rng.normal(0, 3, (5, 7, 11)).astype(want_dtype)
+        got = (want + rng.normal(0, 1e-3, want.shape)).astype(np.float32)
+        rel, max_abs, max_ref = oracle.compare(got, want)
+        d = got.astype(np.float64) - want.astype(np.float64)
+        assert rel == pytest.approx(np.linalg.norm(d.ravel()) / np.linalg.norm(want.astype(np.float64).ravel()), rel=1e-12)
+        assert max_abs == pytest.approx(np.abs(d).max(), rel=1e-12)
+        assert max_ref == pytest.approx(np.abs(want).max(), rel=1e-12)
+        # identical tensors: exactly zero
+        same = want.astype(np.float32)
+        assert oracle.compare(same, same.astype(want_dtype))[:2] == (0.0, 0.0)
+        # one wrong element is seen by both error figures
+        bad = same.copy()
+        bad[2, 3, 4] += 0.5
+        rel1, max1, _ = oracle.compare(bad, same.astype(want_dtype))
+        assert max1 == pytest.approx(0.5, rel=1e-6)
+        assert rel1 == pytest.approx(0.5 / np.linalg.norm(same.astype(np.float64).ravel()), rel=1e-6)
+        # a NaN or an infinity in the result can never pass a bound
+        for poison in (np.nan, np.inf, -np.inf):
+            p = same.copy()
+            p[0, 0, 0] = poison
+            rel2, max2, _ = oracle.compare(p, same.astype(want_dtype))
+            assert not rel2 <= 1e30 and not max2 <= 1e30
 
 
 @pytest.mark.parametrize("quant,bound", [(1, 2e-3), (2, 1.5e-2)])
