@@ -198,6 +198,27 @@ int opencnn_conv_forward_pretransformed(const float *in, const float *Ww, float 
                                         int filt_k);
 
 /*
+ * convolutionForward for callers that cannot allocate device memory and so have no Ww to pass:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No
+ * counterpart in the reference (its caller always allocates Ww, src/openCNN_winograd.cu:310-311).
+ * Same filter transform and fused kernel as convolutionForward (in CHWN, w CRSK, out KHWN,
+ * in_h == in_w, the selected stream and operand precision), but the transformed filter goes
+ * into a workspace inside the library: opencnn_static_workspace_bytes() = 16 MiB of static
+ * device memory per GPU, enough for in_c = filt_k = 512.  The call allocates and frees nothing.
+ *   - opencnn_init() must have run on the current device (hipErrorNotInitialized otherwise): it
+ *     loads the kernels and looks the workspace up, which this call must not do.
+ *   - shapes with opencnn_workspace_bytes(in_c, filt_k) above the limit return
+ *     hipErrorInvalidValue and launch nothing.
+ *   - every call on a GPU uses that GPU's one workspace, whatever the stream: calls on the same
+ *     stream are ordered, calls that overlap in time on one GPU (two streams, two threads) race
+ *     on it and must not be made.  The workspace keeps the last call's transformed filter;
+ *     each call overwrites all of what it reads.
+ */
+int opencnn_conv_forward_static(const float *in, const float *w, float *out, int in_n,
+                                int in_c, int in_h, int in_w, int filt_k);
+size_t opencnn_static_workspace_bytes(void);
+
+/*
  * Bench support, the library-side twin of the reference's timing loop
  * (src/openCNN_winograd.cu:426-444): `warmup` untimed calls, then `iters` back-to-back
  * calls bracketed by HIP events on the selected stream.  Writes mean milliseconds per

@@ -12,6 +12,8 @@ from .binding import (  # noqa: F401
     OpenCNNError,
     convolutionForward,
     conv_forward_pretransformed,
+    conv_forward_static,
+    static_workspace_bytes,
     filter_transform,
     init,
     lib,
@@ -56,6 +58,7 @@ __all__ = [
     "OpenCNNError",
     "convolutionForward",
     "conv_forward_pretransformed",
+    "conv_forward_static",
     "filter_transform",
     "init",
     "last_kernel",

@@ -50,6 +50,9 @@ EXPORTED_SYMBOLS = {
     "opencnn_filter_transform": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int]),
     "opencnn_conv_forward_pretransformed": (
         _c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int]),
+    "opencnn_conv_forward_static": (
+        _c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int]),
+    "opencnn_static_workspace_bytes": (ctypes.c_size_t, []),
     "opencnn_nchw_to_chwn": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int]),
     "opencnn_khwn_to_nkhw": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int]),
     "opencnn_kcrs_to_crsk": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int]),
@@ -145,7 +148,7 @@ def _dev_f32(buf, what: str) -> int:
 
 def _check(func: str, status: int) -> None:
     if status != 0:
-        detail = lib().opencnn_last_error().decode() if status == 1 else ""
+        detail = lib().opencnn_last_error().decode() if status in (1, 3) else ""
         raise OpenCNNError(func, status, detail)
 
 
@@ -231,6 +234,17 @@ def conv_forward_pretransformed(x, Ww, y, in_n, in_c, in_h, in_w, filt_k) -> Non
     _check("opencnn_conv_forward_pretransformed", lib().opencnn_conv_forward_pretransformed(
         _dev_f32(x, "input"), _dev_f32(Ww, "workspace"), _dev_f32(y, "output"), in_n, in_c,
         in_h, in_w, filt_k))
+
+
+def conv_forward_static(x, w, y, in_n, in_c, in_h, in_w, filt_k) -> None:
+    """convolutionForward on the library's static workspace (allocates nothing; needs init())."""
+    _check("opencnn_conv_forward_static", lib().opencnn_conv_forward_static(
+        _dev_f32(x, "input"), _dev_f32(w, "filter"), _dev_f32(y, "output"), in_n, in_c, in_h,
+        in_w, filt_k))
+
+
+def static_workspace_bytes() -> int:
+    return lib().opencnn_static_workspace_bytes()
 
 
 def nchw_to_chwn(src, dst, n, c, h, w) -> None:

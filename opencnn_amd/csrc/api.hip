@@ -24,6 +24,7 @@ std::atomic<int> g_balance{1};
 std::atomic<int> g_precision{OPENCNN_F32};
 std::atomic<long long*> g_timeline{nullptr};
 std::atomic<size_t> g_timeline_bytes{0};
+std::atomic<bool> g_device_ready[64];  // set-up of asm_kernels() done on that device
 
 // Compute units of the current device (cached per device index).
 int compute_units(int* out) {
@@ -47,6 +48,11 @@ thread_local const char* t_last_kernel = "";
 extern "C" const char opencnn_wino_f32_asm_hsaco[];
 extern "C" const char opencnn_wino_h16_asm_hsaco[];  // gen_wino_h16_asm.py
 
+// Workspace of opencnn_conv_forward_static: the transformed filter of one call.  One copy per
+// GPU the library runs on, held until the process ends; every call on a GPU shares it.
+constexpr size_t kScratchBytes = 16u << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
 struct AsmKernels {
   hipModule_t module = nullptr, module_h16 = nullptr;
   hipFunction_t kw2 = nullptr, kw4 = nullptr, kw2_ragged = nullptr, kw4_ragged = nullptr;
@@ -54,6 +60,7 @@ struct AsmKernels {
   hipFunction_t f16_kw4 = nullptr, bf16_kw4 = nullptr, f16_kw4_ragged = nullptr, bf16_kw4_ragged = nullptr;
   hipFunction_t f16_kw4_packed = nullptr, bf16_kw4_packed = nullptr;
   unsigned* split_sync = nullptr;  // device address of g_split_sync (all sets) on this device
+  float* scratch = nullptr;        // device address of `scratch` on this device
   bool ready = false;
 };
 
@@ -84,11 +91,25 @@ int asm_kernels(const AsmKernels** out) {
     if ((e = hipModuleGetFunction(&k.bf16_kw4_packed, k.module_h16, "wino_bf16_asm_kw4_packed")) != hipSuccess) return (int)e;
     if ((e = hipGetSymbolAddress(reinterpret_cast<void**>(&k.split_sync), HIP_SYMBOL(opencnn::g_split_sync))) != hipSuccess)
       return (int)e;
+    // the array's name is a host-side stand-in; this is its address on the current device
+    if ((e = hipGetSymbolAddress(reinterpret_cast<void**>(&k.scratch), HIP_SYMBOL(scratch))) != hipSuccess)
+      return (int)e;
     // 64 KB of dynamic LDS for KW = 2 is the default limit exactly; nothing to raise
     k.ready = true;
+    g_device_ready[dev].store(true);
   }
   *out = &k;
   return 0;
+}
+
+// The same record if opencnn_init (or a launch) has set this device up already, else null: for
+// callers that must not load code objects or allocate.
+const AsmKernels* asm_kernels_if_ready() {
+  const AsmKernels* ak = nullptr;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  if (!g_device_ready[dev].load()) return nullptr;
+  return asm_kernels(&ak) == 0 ? ak : nullptr;
 }
 
 // The split-merge flags come in kSyncSets sets; every stream that launches gets a set of its own
@@ -781,6 +802,25 @@ int convolutionForward(float* k, int in_h, int in_w, float* w, int out_h, int ou
                                     tiles_dim, in_n, tile_size, in_c, filt_k, filt_c, filt_h,
                                     filt_w, alpha, m);
 }
+
+int opencnn_conv_forward_static(const float* in, const float* w, float* out, int in_n, int in_c,
+                                int in_h, int in_w, int filt_k) {
+  REQUIRE(in != nullptr && w != nullptr && out != nullptr);
+  REQUIRE(in_h == in_w);  // as convolutionForward
+  if (int e = check_conv_shape(in_n, in_c, in_h, in_w, filt_k)) return e;
+  if (opencnn_workspace_bytes(in_c, filt_k) > kScratchBytes)
+    return fail("transformed filter exceeds the static workspace (opencnn_static_workspace_bytes)");
+  const AsmKernels* ak = asm_kernels_if_ready();
+  if (ak == nullptr) {
+    t_last_error = "opencnn_init() has not run on this device";
+    return (int)hipErrorNotInitialized;
+  }
+  hipStream_t st = g_stream.load();
+  if (int e = launch_fx(w, ak->scratch, filt_k, in_c, OPENCNN_FILTER_CRSK, OPENCNN_WW_MFMA, st)) return e;
+  return launch_main(in, ak->scratch, out, in_n, in_c, in_h, in_w, filt_k, st);
+}
+
+size_t opencnn_static_workspace_bytes(void) { return kScratchBytes; }
 
 int opencnn_time_forward(const float* in, const float* w, float* out, float* Ww, int in_n,
                          int in_c, int in_h, int in_w, int filt_k, int warmup, int iters,
