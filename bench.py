@@ -38,15 +38,29 @@ LAYERS = {
 FP32_LAYERS = [k for k in LAYERS if not k.startswith("reduced")]
 DEFAULT_WORKLOAD = "resnet_n64_c64_h56_k64"
 
-# HBM bytes per launch of the fused kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# (profiles/), or None where not measured yet.
-MEASURED_TRAFFIC_BYTES = {
-    "resnet_n64_c64_h56_k64": 214.3e6,
-    "resnet_n128_c128_h28_k128": 261.2e6,
-    "deep_n128_c256_h14_k256": 249.7e6,
-    "deep_n128_c512_h7_k512": 112.7e6,
-    "reduced_n128_c256_h14_k256_f16": 164.5e6,
-}
+# HBM bytes per launch of the fused kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs:
+# profiles/traffic.json, written when the profiles are refreshed, with the commit the kernels
+# were measured at (a later change of a kernel makes its entry stale: compare with HEAD).
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+
+
+def measured_traffic(key):
+    """(bytes per launch, commit they were measured at), or (None, None)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            table = json.load(f)
+    except (OSError, ValueError):
+        return None, None
+    row = table.get("workloads", {}).get(key)
+    return (row["traffic_bytes"], table.get("commit")) if row else (None, None)
+
+
+def custom_layer(spec):
+    """--shape N,C,H,K -> a workload of that shape (uniform[-1,1] input, He-init filters)."""
+    n, c, h, k = (int(v) for v in spec.split(","))
+    name = f"custom_n{n}_c{c}_h{h}_k{k}"
+    LAYERS[name] = (n, c, h, k, (-1.0, 1.0), "he")
+    return name
 
 
 def work(N, C, H, K):
@@ -81,10 +95,25 @@ class Layer:
                                     o.K * o.N * o.H * o.H, o.td, o.N, 4, o.td * 4, o.C, o.K,
                                     o.C, 3, 3, 4, 2)
 
-    def kernel_times(self, warmup, iters):
+    def kernel_times(self, warmup, iters, parts=("total", "main", "fx")):
         """HIP-event mean ms per call on the library's stream: (fx+main, main, fx)."""
         return self.ocn.time_forward(self.x, self.w, self.y, self.ws, self.N, self.C, self.H,
-                                     self.H, self.K, warmup=warmup, iters=iters)
+                                     self.H, self.K, warmup=warmup, iters=iters, parts=parts)
+
+
+def from_idle(torch, lay, flops_mfma, peak, idle_s=0.5):
+    """The reference's own protocol (src/openCNN_winograd.cu:426-444): one warm-up call, then 100
+    back-to-back calls between two events, starting from an idle device - no settle phase.  Once
+    for the whole call (filter transform + fused kernel) and, after another idle period, once
+    for the fused kernel alone."""
+    torch.cuda.synchronize()
+    time.sleep(idle_s)
+    total, _, _ = lay.kernel_times(1, 100, parts=("total",))
+    time.sleep(idle_s)
+    _, main, _ = lay.kernel_times(1, 100, parts=("main",))
+    return {"protocol": "0.5 s idle, 1 warm-up call, 100 timed calls (HIP events), as the reference's bench",
+            "ms_per_step": total, "ms_fused_kernel": main,
+            "frac": flops_mfma / (main * 1e-3) / 1e12 / peak}
 
 
 def settle(torch, lay, ms):
@@ -307,6 +336,9 @@ def main():
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(LAYERS))
+    ap.add_argument("--shape", default=None, metavar="N,C,H,K",
+                    help="time a layer of this shape instead of a named workload (for profiles of "
+                         "shapes outside the benchmark set)")
     ap.add_argument("--operands", default="f32", choices=["f32", "f16", "bf16"],
                     help="GEMM operand precision of the timed workload (fp32 transforms and "
                          "accumulation in every case); the default is the reference's fp32")
@@ -339,6 +371,8 @@ def main():
         sys.exit("bench.py: no GPU visible")
     ocn.init()
 
+    if args.shape:
+        args.workload = custom_layer(args.shape)
     layer = Layer(ocn, torch, args.workload)
     fd, fm, bmin = work(layer.N, layer.C, layer.H, layer.K)
     reduced = args.operands != "f32"
@@ -346,6 +380,7 @@ def main():
         ocn.set_operand_precision(ocn.F16 if args.operands == "f16" else ocn.BF16)
     peak = PEAK_F16_MFMA_TFLOPS if reduced else PEAK_FP32_MFMA_TFLOPS
 
+    idle = from_idle(torch, layer, fm, peak)  # first: nothing has run on the device yet
     settle(torch, layer, args.settle_ms)
     for _ in range(args.warmup):
         layer.step()
@@ -360,8 +395,11 @@ def main():
     # dominant kernel, HIP events on the launch stream, same number of launches
     _, ms_main, ms_fx = layer.kernel_times(args.warmup, args.steps)
     achieved = fm / (ms_main * 1e-3) / 1e12
-    traffic = MEASURED_TRAFFIC_BYTES.get(layer.name + ("_" + args.operands if reduced else ""))
+    traffic, traffic_commit = measured_traffic(layer.name + ("_" + args.operands if reduced else ""))
+    kernel_name = ocn.last_kernel()
+    grid, flag_set = ocn.last_launch()
     ocn.set_operand_precision(ocn.F32)
+    ocn.check_status()  # raises if any launch so far gave up a hand-over between workgroups
 
     out = {
         "metric": "effective TFLOP/s (direct-conv FLOPs 2*N*K*C*H*W*9) of one 3x3 layer, "
@@ -382,14 +420,14 @@ def main():
                    "W": layer.H, "K": layer.K, "pad": 1, "stride": 1,
                    "layout": "CHWN in, CRSK filters, KHWN out"},
         "roofline": {
-            "kernel": ("wino_f16_asm_kw4 / wino_bf16_asm_kw4" if reduced else "wino_f32_asm_kw2 / wino_f32_asm_kw4") +
-                      " (fused Winograd kernel, hand-scheduled assembly)",
+            "kernel": kernel_name + " (fused Winograd kernel), %d workgroups, flag set %d" % (grid, flag_set),
             "bound": "mfma",
             "achieved": achieved,
             "peak": peak,
             "unit": "TFLOP/s",
             "frac": achieved / peak,
             "traffic": traffic,
+            "traffic_commit": traffic_commit,
             "flops_per_launch": fm,
             "ms_per_launch": ms_main,
             "hbm_min_bytes": bmin,
@@ -399,7 +437,19 @@ def main():
             "hbm_frac_of_peak_measured_traffic": (traffic / (ms_main * 1e-3) / 1e9 / PEAK_HBM_GBS) if traffic else None,
             "fx_ms_per_launch": ms_fx,
         },
+        "from_idle": idle,
     }
+    if reduced:
+        # The fp16 / bf16 matrix pipe is not what bounds this kernel: a 16-channel unit needs 512
+        # MFMA cycles but 96 KB of operands per workgroup (64 KB of transformed filters, 32 KB of
+        # fp32 patches) through the compute unit's 64 B/clk vector-memory path: 1536 cycles.
+        units = ((layer.H + 1) // 2) ** 2 * ((layer.N + 31) // 32) * ((layer.K + 127) // 128) * ((layer.C + 15) // 16)
+        roof_ms = units * 1536 / 256 / 2.4e9 * 1e3
+        out["roofline"]["operand_delivery_roof"] = {
+            "what": "vector-memory path of a compute unit, 64 B/clk: 96 KB per (workgroup tile, 16-channel unit) "
+                    "= 1536 cycles against 512 cycles of MFMA",
+            "ms_at_roof": roof_ms, "frac": roof_ms / ms_main,
+            "mfma_frac_at_this_roof": fm / (roof_ms * 1e-3) / 1e12 / peak}
 
     if not args.no_cpu:
         from oracle import oracle

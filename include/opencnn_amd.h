@@ -5,10 +5,13 @@
  * allocated on the current HIP device (any float-aligned address, e.g. a slice of a larger
  * allocation); the library allocates no tensors or workspaces.  Its
  * state between calls is the process-wide settings of the opencnn_set_* calls below (stream,
- * kernel variant, balanced split, operand precision), the code objects of its assembly kernels
- * (embedded in the library, loaded once per device by opencnn_init or the first launch) and
- * 256 KB of static device memory that the balanced split uses to hand tiles over between
- * workgroups (eight sets of flags, one per stream; zero between launches).
+ * kernel variant, balanced split, operand precision; opencnn_conv_forward_desc takes all of
+ * them per call instead), the code objects of its assembly kernels (embedded in the library,
+ * loaded once per device by opencnn_init or the first launch), 1.5 MB of static device memory
+ * that the balanced split uses to hand tiles over between workgroups (48 sets of flags, zero
+ * between launches; see opencnn_set_balanced_split), 200 bytes of pinned host memory per device
+ * that the kernels report a failed hand-over in (opencnn_check_status), and a host-side record of
+ * the transformed filters it wrote (opencnn_filter_transform).
  * All entry points return a hipError_t value as int (0 == hipSuccess); launches are
  * asynchronous on the selected stream, exactly like the reference, which returns
  * cudaGetLastError() right after its two launches
@@ -56,7 +59,8 @@ enum {
  * and 16 channels (opencnn_workspace_bytes covers both precisions).  Any in_n, in_c, filt_k.
  * Tensors in HBM stay fp32.
  * opencnn_filter_transform(..., OPENCNN_WW_MFMA) and the fused kernel must run under the same
- * setting.
+ * setting: the library remembers what it wrote to a Ww address and the fused kernel returns
+ * hipErrorInvalidValue for a buffer written under another precision (see opencnn_filter_transform).
  */
 enum { OPENCNN_F32 = 0, OPENCNN_F16 = 1, OPENCNN_BF16 = 2 };
 int opencnn_set_operand_precision(int precision);
@@ -165,13 +169,57 @@ int opencnn_set_kernel_variant(int variant);
  * device state per wave.  Results stay independent of timing (two addends commute).  The same
  * hand-over serves layers with tiles for at most half of the compute units (small batches on
  * deep layers): every tile is cut among two or four workgroups, and the parts of
- * its channel sum are passed from workgroup to workgroup in a fixed order.  That
- * state exists once per stream for the first eight streams that launch (calls on different
- * streams may overlap in time); calls on further streams run without the split.  Pass 0 to
- * turn it off altogether.  No counterpart in the reference, whose grid is one block per tile
+ * its channel sum are passed from workgroup to workgroup in a fixed order.  Pass 0 to turn
+ * it off altogether.  No counterpart in the reference, whose grid is one block per tile
  * (src/convolutionForward_32x64x8.cu:281).
+ *
+ * Launches that may overlap in time must not share that state, so it exists in sets:
+ *   - every stream that launches directly holds one of 32 sets.  The library never touches a
+ *     stream it is not asked to launch on (its handle may be stale), so a set only changes
+ *     hands on the library's own evidence: from the moment a 33rd stream launches, every launch
+ *     is followed by an event (hipEventRecord, about a microsecond), and a stream without a set
+ *     takes over the set used longest ago whose event has completed.  Until one has, its
+ *     launches run without the split (slower, same results; opencnn_last_launch tells).
+ *     opencnn_release_stream(stream) waits for a stream and gives its set back at once, e.g.
+ *     before the stream is destroyed.
+ *   - launches recorded in a stream capture hold one of 16 further sets per (capture, stream)
+ *     for the life of the process, since the graph may be replayed at any time on any stream;
+ *     the seventeenth runs without the split.  Two executable graphs instantiated from one
+ *     capture share its set and must not run at the same time.
+ *   - a caller that wants neither limit passes flag storage of its own in
+ *     opencnn_conv_desc.split_flags.
  */
 int opencnn_set_balanced_split(int enable);
+int opencnn_release_stream(void *stream);
+
+/*
+ * What this thread's last successful fused-kernel launch looked like: its number of workgroups
+ * and its set of split-merge flags (0..47 a set of the library, 48 the caller's storage, -1
+ * none: the split was off, not needed by any kernel that could run, or no set was free).
+ * Either pointer may be NULL.  For tests and logs; no counterpart in the reference.
+ */
+int opencnn_last_launch(int *workgroups, int *flag_set);
+
+/*
+ * A kernel's wait for another workgroup's partial tile is bounded (about a second), so that
+ * no bug and no workgroup that fails to become resident can hang the GPU.  A wave that gives up
+ * finishes normally, but its launch's output is wrong; it reports that in a status word of the
+ * launch's flag set, in host memory.  The library reads that word (no copy, no
+ * synchronisation) at the next call that uses the same flag set: that call launches nothing
+ * but a kernel that clears the flags, and returns hipErrorLaunchFailure with opencnn_last_error()
+ * saying so; the call after it works again.  opencnn_check_status() does the same check for all
+ * flag sets of the current device at once: call it after synchronising (hipDeviceSynchronize
+ * or the streams in use) to learn whether every launch so far, graph replays included, handed
+ * its tiles over; it returns 0 or hipErrorLaunchFailure (and has then cleared the library's
+ * flag sets; flag storage of a caller is the caller's to clear).
+ * The reference has no hand-over and no such state (one block per tile,
+ * src/convolutionForward_32x64x8.cu:281).
+ *
+ * opencnn_set_wait_limit: the number of polls after which a wait gives up, for tests of this
+ * path (0 restores the default of 2^20 polls).
+ */
+int opencnn_check_status(void);
+int opencnn_set_wait_limit(unsigned polls);
 
 /*
  * The reference's FX kernel as a call of its own (src/FX_m2.cu:51-91, launched at
@@ -181,9 +229,17 @@ int opencnn_set_balanced_split(int enable);
  *                  OPENCNN_WW_REFERENCE, opencnn_workspace_bytes() for OPENCNN_WW_MFMA
  * OPENCNN_WW_REFERENCE output is bit-identical to the reference's arithmetic order
  * (only additions and multiplications by 0.5).
+ *
+ * The library remembers, per device and Ww address (the 64 most recent), the layout, operand
+ * precision and filter shape of what it wrote there.  The fused kernel checks a Ww it is given
+ * against that record and returns hipErrorInvalidValue on a mismatch (a 2-byte Ww read as floats
+ * would give garbage without any other sign); an address without a record is taken as it is.
+ * A caller that fills such an address by other means (a copy of a transformed filter saved
+ * elsewhere) drops the stale record with opencnn_forget_workspace(Ww).
  */
 int opencnn_filter_transform(const float *w, float *Ww, int filt_k, int filt_c,
                              int filter_layout, int ww_layout);
+int opencnn_forget_workspace(const void *Ww);
 
 /*
  * The reference's Winograd_kernel as a call of its own
@@ -196,6 +252,46 @@ int opencnn_filter_transform(const float *w, float *Ww, int filt_k, int filt_c,
 int opencnn_conv_forward_pretransformed(const float *in, const float *Ww, float *out,
                                         int in_n, int in_c, int in_h, int in_w,
                                         int filt_k);
+
+/*
+ * One call with all of its settings: what the process-wide opencnn_set_* calls select for the
+ * other entry points, per call, so that threads can use different streams, precisions and
+ * kernels at the same time.  No counterpart in the reference (one thread, the null stream,
+ * src/openCNN_winograd.cu:426-444).
+ *   struct_size        sizeof(opencnn_conv_desc) (other values return hipErrorInvalidValue)
+ *   in, out            CHWN input, KHWN output; in_h and in_w may differ
+ *   filter             3x3 filters in filter_layout, or NULL
+ *   Ww                 opencnn_workspace_bytes(in_c, filt_k) bytes.  With a filter: scratch, as
+ *                      in convolutionForward (the filter transform runs first).  With
+ *                      filter == NULL: a transformed filter that an earlier call on the same
+ *                      stream left there under the same operand_precision (the split API).
+ *   operand_precision  OPENCNN_F32 / F16 / BF16;  kernel_variant OPENCNN_KERNEL_*;
+ *   balanced_split     0 / 1;  stream  a hipStream_t, NULL = the null stream
+ *   split_flags        NULL (the library's flag sets, see opencnn_set_balanced_split), or
+ *                      split_flags_bytes >= opencnn_split_flags_bytes() of device memory that the
+ *                      caller zeroed once: the hand-over state of this call.  Calls that share
+ *                      one such buffer must not overlap in time; calls with different buffers may,
+ *                      on any number of streams and graphs.
+ * A zero-initialised struct with struct_size, the pointers and the shape filled in selects
+ * the defaults except for balanced_split, which a caller who wants the default sets to 1.
+ */
+typedef struct opencnn_conv_desc {
+  size_t struct_size;
+  const float *in;
+  const float *filter;
+  float *out;
+  void *Ww;
+  int in_n, in_c, in_h, in_w, filt_k;
+  int filter_layout;
+  int operand_precision;
+  int kernel_variant;
+  int balanced_split;
+  void *stream;
+  void *split_flags;
+  size_t split_flags_bytes;
+} opencnn_conv_desc;
+int opencnn_conv_forward_desc(const opencnn_conv_desc *desc);
+size_t opencnn_split_flags_bytes(void);
 
 /*
  * convolutionForward for callers that cannot allocate device memory and so have no Ww to pass:
@@ -244,7 +340,8 @@ int opencnn_set_timeline_buffer(long long *device_buffer, size_t bytes);
  * kernel (src/openCNN_winograd.cu:147-153) as used at :230 (NCHW input -> CHWN) and :235 (KCRS
  * filters -> CRSK), plus the way back for the result (KHWN -> NKHW, i.e. NCHW with K channels),
  * which the reference only does implicitly inside its checker's index map (:185-186).
- * data_cpy is limited to C <= 1024 by its launch shape; these are not.
+ * data_cpy is limited to C <= 1024 by its launch shape; these take any tensor below 2^31
+ * elements.
  */
 int opencnn_nchw_to_chwn(const float *src, float *dst, int n, int c, int h, int w);
 int opencnn_khwn_to_nkhw(const float *src, float *dst, int n, int k, int h, int w);

@@ -73,7 +73,27 @@ EXPORTED_SYMBOLS = {
     ),
     "opencnn_last_error": (ctypes.c_char_p, []),
     "opencnn_last_kernel": (ctypes.c_char_p, []),
+    "opencnn_last_launch": (_c_int, [ctypes.POINTER(_c_int), ctypes.POINTER(_c_int)]),
+    "opencnn_check_status": (_c_int, []),
+    "opencnn_release_stream": (_c_int, [_c_void_p]),
+    "opencnn_set_wait_limit": (_c_int, [ctypes.c_uint]),
+    "opencnn_forget_workspace": (_c_int, [_c_void_p]),
+    "opencnn_conv_forward_desc": (_c_int, [_c_void_p]),
+    "opencnn_split_flags_bytes": (ctypes.c_size_t, []),
 }
+
+
+class ConvDesc(ctypes.Structure):
+    """opencnn_conv_desc of include/opencnn_amd.h."""
+
+    _fields_ = [
+        ("struct_size", ctypes.c_size_t),
+        ("in_", _c_void_p), ("filter", _c_void_p), ("out", _c_void_p), ("Ww", _c_void_p),
+        ("in_n", _c_int), ("in_c", _c_int), ("in_h", _c_int), ("in_w", _c_int), ("filt_k", _c_int),
+        ("filter_layout", _c_int), ("operand_precision", _c_int), ("kernel_variant", _c_int),
+        ("balanced_split", _c_int),
+        ("stream", _c_void_p), ("split_flags", _c_void_p), ("split_flags_bytes", ctypes.c_size_t),
+    ]
 
 
 class OpenCNNError(RuntimeError):
@@ -148,7 +168,8 @@ def _dev_f32(buf, what: str) -> int:
 
 def _check(func: str, status: int) -> None:
     if status != 0:
-        detail = lib().opencnn_last_error().decode() if status in (1, 3) else ""
+        # hipErrorInvalidValue, hipErrorNotInitialized, hipErrorLaunchFailure: set by the library itself
+        detail = lib().opencnn_last_error().decode() if status in (1, 3, 719) else ""
         raise OpenCNNError(func, status, detail)
 
 
@@ -159,6 +180,68 @@ def init() -> None:
 def last_kernel() -> str:
     """Name of the fused kernel this thread's last successful launch used."""
     return lib().opencnn_last_kernel().decode()
+
+
+def last_launch():
+    """(workgroups, flag set) of this thread's last successful fused-kernel launch; flag set -1 =
+    launched without the split."""
+    grid, flag_set = _c_int(0), _c_int(0)
+    _check("opencnn_last_launch", lib().opencnn_last_launch(ctypes.byref(grid), ctypes.byref(flag_set)))
+    return grid.value, flag_set.value
+
+
+def check_status() -> None:
+    """Raises OpenCNNError (hipErrorLaunchFailure, 719) if a launch on the current device gave up
+    waiting for a partial tile since the last check; call after synchronising."""
+    _check("opencnn_check_status", lib().opencnn_check_status())
+
+
+def release_stream(stream) -> None:
+    """Wait for `stream` and give its set of split-merge flags back."""
+    handle = 0 if stream is None else getattr(stream, "cuda_stream", stream)
+    _check("opencnn_release_stream", lib().opencnn_release_stream(handle))
+
+
+def set_wait_limit(polls: int) -> None:
+    """Polls after which a kernel's wait for a partial tile gives up (0: the default)."""
+    _check("opencnn_set_wait_limit", lib().opencnn_set_wait_limit(polls))
+
+
+def split_flags_bytes() -> int:
+    return lib().opencnn_split_flags_bytes()
+
+
+def forget_workspace(Ww) -> None:
+    _check("opencnn_forget_workspace", lib().opencnn_forget_workspace(_ptr(Ww)))
+
+
+def _workspace(buf, filt_c: int, filt_k: int) -> int:
+    """Address of a Ww buffer after checking that it holds opencnn_workspace_bytes()."""
+    if hasattr(buf, "numel"):
+        have, need = buf.numel() * buf.element_size(), workspace_bytes(filt_c, filt_k)
+        if have < need:
+            raise ValueError(f"workspace holds {have} bytes, opencnn_workspace_bytes({filt_c}, {filt_k}) = {need}")
+    return _dev_f32(buf, "workspace")
+
+
+def conv_forward_desc(x, w, y, Ww, in_n, in_c, in_h, in_w, filt_k, *, filter_layout=FILTER_CRSK,
+                      precision=F32, variant=KERNEL_AUTO, balanced_split=True, stream=None,
+                      split_flags=None) -> None:
+    """opencnn_conv_forward_desc: one call with its own settings.  `w` None = Ww holds a
+    transformed filter already; `split_flags` a zeroed CUDA tensor of split_flags_bytes() or None."""
+    d = ConvDesc()
+    d.struct_size = ctypes.sizeof(ConvDesc)
+    d.in_, d.out = _dev_f32(x, "input"), _dev_f32(y, "output")
+    d.filter = None if w is None else _dev_f32(w, "filter")
+    d.Ww = _workspace(Ww, in_c, filt_k)
+    d.in_n, d.in_c, d.in_h, d.in_w, d.filt_k = in_n, in_c, in_h, in_w, filt_k
+    d.filter_layout, d.operand_precision, d.kernel_variant = filter_layout, precision, variant
+    d.balanced_split = 1 if balanced_split else 0
+    d.stream = None if stream is None else getattr(stream, "cuda_stream", stream)
+    if split_flags is not None:
+        d.split_flags = _ptr(split_flags)
+        d.split_flags_bytes = split_flags.numel() * split_flags.element_size()
+    _check("opencnn_conv_forward_desc", lib().opencnn_conv_forward_desc(ctypes.byref(d)))
 
 
 def tiles_dim(in_w: int) -> int:
@@ -219,20 +302,20 @@ def convolutionForward(k, in_h, in_w, w, out_h, out_w, out_n, out_c, C, Ww, n, t
     ``k`` CHWN input, ``w`` CRSK filters, ``C`` KHWN output, ``Ww`` workspace."""
     _check("convolutionForward", lib().convolutionForward(
         _dev_f32(k, "input"), in_h, in_w, _dev_f32(w, "filter"), out_h, out_w, out_n, out_c,
-        _dev_f32(C, "output"), _dev_f32(Ww, "workspace"), n, tiles_dim, in_n, tile_size,
+        _dev_f32(C, "output"), _workspace(Ww, filt_c, filt_k), n, tiles_dim, in_n, tile_size,
         elems_dim, in_c, filt_k, filt_c, filt_h, filt_w, alpha, m))
 
 
 def filter_transform(w, Ww, filt_k, filt_c, filter_layout=FILTER_CRSK,
                      ww_layout=WW_REFERENCE) -> None:
+    ww = _workspace(Ww, filt_c, filt_k) if ww_layout == WW_MFMA else _dev_f32(Ww, "workspace")
     _check("opencnn_filter_transform", lib().opencnn_filter_transform(
-        _dev_f32(w, "filter"), _dev_f32(Ww, "workspace"), filt_k, filt_c, filter_layout,
-        ww_layout))
+        _dev_f32(w, "filter"), ww, filt_k, filt_c, filter_layout, ww_layout))
 
 
 def conv_forward_pretransformed(x, Ww, y, in_n, in_c, in_h, in_w, filt_k) -> None:
     _check("opencnn_conv_forward_pretransformed", lib().opencnn_conv_forward_pretransformed(
-        _dev_f32(x, "input"), _dev_f32(Ww, "workspace"), _dev_f32(y, "output"), in_n, in_c,
+        _dev_f32(x, "input"), _workspace(Ww, in_c, filt_k), _dev_f32(y, "output"), in_n, in_c,
         in_h, in_w, filt_k))
 
 
@@ -259,13 +342,15 @@ def kcrs_to_crsk(src, dst, k, c) -> None:
     _check("opencnn_kcrs_to_crsk", lib().opencnn_kcrs_to_crsk(_dev_f32(src, "src"), _dev_f32(dst, "dst"), k, c))
 
 
-def time_forward(x, w, y, Ww, in_n, in_c, in_h, in_w, filt_k, warmup=1, iters=100):
-    """Mean ms per call: (filter transform + fused kernel, fused kernel, filter transform)."""
+def time_forward(x, w, y, Ww, in_n, in_c, in_h, in_w, filt_k, warmup=1, iters=100,
+                 parts=("total", "main", "fx")):
+    """Mean ms per call: (filter transform + fused kernel, fused kernel, filter transform); only
+    the loops named in `parts` run, the others come back as 0."""
     t = [ctypes.c_float(0.0) for _ in range(3)]
+    ref = [ctypes.byref(t[i]) if name in parts else None for i, name in enumerate(("total", "main", "fx"))]
     _check("opencnn_time_forward", lib().opencnn_time_forward(
         _dev_f32(x, "input"), _dev_f32(w, "filter"), _dev_f32(y, "output"),
-        _dev_f32(Ww, "workspace"), in_n, in_c, in_h, in_w, filt_k, warmup, iters,
-        ctypes.byref(t[0]), ctypes.byref(t[1]), ctypes.byref(t[2])))
+        _workspace(Ww, in_c, filt_k), in_n, in_c, in_h, in_w, filt_k, warmup, iters, *ref))
     return t[0].value, t[1].value, t[2].value
 
 

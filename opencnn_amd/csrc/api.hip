@@ -24,7 +24,29 @@ std::atomic<int> g_balance{1};
 std::atomic<int> g_precision{OPENCNN_F32};
 std::atomic<long long*> g_timeline{nullptr};
 std::atomic<size_t> g_timeline_bytes{0};
-std::atomic<bool> g_device_ready[64];  // set-up of asm_kernels() done on that device
+std::atomic<bool> g_device_ready[64];  // set-up of device_state() done on that device
+// Polls after which a kernel's wait for a split-merge flag gives up (about a second).
+constexpr unsigned kDefaultWaitPolls = 1u << 20;
+std::atomic<unsigned> g_wait_polls{kDefaultWaitPolls};
+
+// The settings of one call: what the opencnn_set_* calls select for the entry points that take no
+// descriptor, or the fields of an opencnn_conv_desc.
+struct CallSettings {
+  hipStream_t stream = nullptr;
+  int variant = OPENCNN_KERNEL_AUTO;
+  int precision = OPENCNN_F32;
+  bool balance = true;
+  unsigned* caller_flags = nullptr;  // split-merge flags the caller owns, or null: a set of the library's
+};
+
+CallSettings process_settings() {
+  CallSettings c;
+  c.stream = g_stream.load();
+  c.variant = g_variant.load();
+  c.precision = g_precision.load();
+  c.balance = g_balance.load() != 0;
+  return c;
+}
 
 // Compute units of the current device (cached per device index).
 int compute_units(int* out) {
@@ -43,6 +65,8 @@ int compute_units(int* out) {
 }
 thread_local const char* t_last_error = "";
 thread_local const char* t_last_kernel = "";
+thread_local int t_last_grid = 0;       // workgroups of this thread's last fused-kernel launch
+thread_local int t_last_flag_set = -1;  // its flag set: -1 none, kSyncSets = the caller's storage
 
 // ---- hand-scheduled assembly kernels (gen_wino_f32_asm.py), loaded from the embedded code object
 extern "C" const char opencnn_wino_f32_asm_hsaco[];
@@ -53,7 +77,21 @@ extern "C" const char opencnn_wino_h16_asm_hsaco[];  // gen_wino_h16_asm.py
 constexpr size_t kScratchBytes = 16u << 20;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
-struct AsmKernels {
+// Who holds a set of split-merge flags.
+struct FlagSetOwner {
+  bool used = false;
+  hipStream_t stream = nullptr;
+  unsigned long long capture_id = 0;  // graph sets: the stream capture the launches were recorded in
+  unsigned long long last_use = 0;
+  int calls_in_flight = 0;     // host calls between taking the set and having launched on it
+  hipEvent_t idle = nullptr;   // eager sets under pressure: recorded behind the set's last launch
+  bool idle_recorded = false;
+};
+
+// Index of the status word of flag storage that a caller passed in a descriptor.
+constexpr int kCallerSet = opencnn::kSyncSets;
+
+struct DeviceState {
   hipModule_t module = nullptr, module_h16 = nullptr;
   hipFunction_t kw2 = nullptr, kw4 = nullptr, kw2_ragged = nullptr, kw4_ragged = nullptr;
   hipFunction_t kw2_packed = nullptr, kw4_packed = nullptr;
@@ -61,19 +99,28 @@ struct AsmKernels {
   hipFunction_t f16_kw4_packed = nullptr, bf16_kw4_packed = nullptr;
   unsigned* split_sync = nullptr;  // device address of g_split_sync (all sets) on this device
   float* scratch = nullptr;        // device address of `scratch` on this device
+  // One status word per flag set plus one for callers' own flag storage, in pinned host memory
+  // that the GPU writes directly: a wave that gives up waiting for a flag stores 1 there, and
+  // the host sees it at its next call without a copy or a synchronisation.
+  volatile unsigned* status_host = nullptr;
+  unsigned* status_dev = nullptr;
+  FlagSetOwner owners[opencnn::kSyncSets];
+  unsigned long long clock = 0;
+  bool pressure = false;  // more streams have launched than there are eager sets
+  std::mutex flag_mu;
   bool ready = false;
 };
 
 // Loaded once per device, with that device current.
-int asm_kernels(const AsmKernels** out) {
-  static AsmKernels per_device[64];
+int device_state(DeviceState** out) {
+  static DeviceState per_device[64];
   static std::mutex mu;
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return (int)e;
   if (dev < 0 || dev >= 64) return (int)hipErrorInvalidDevice;
   std::lock_guard<std::mutex> lock(mu);
-  AsmKernels& k = per_device[dev];
+  DeviceState& k = per_device[dev];
   if (!k.ready) {
     if ((e = hipModuleLoadData(&k.module, opencnn_wino_f32_asm_hsaco)) != hipSuccess) return (int)e;
     if ((e = hipModuleGetFunction(&k.kw2, k.module, "wino_f32_asm_kw2")) != hipSuccess) return (int)e;
@@ -94,6 +141,13 @@ int asm_kernels(const AsmKernels** out) {
     // the array's name is a host-side stand-in; this is its address on the current device
     if ((e = hipGetSymbolAddress(reinterpret_cast<void**>(&k.scratch), HIP_SYMBOL(scratch))) != hipSuccess)
       return (int)e;
+    void* host = nullptr;
+    void* dev_view = nullptr;
+    if ((e = hipHostMalloc(&host, (kCallerSet + 1) * sizeof(unsigned), hipHostMallocMapped)) != hipSuccess) return (int)e;
+    std::memset(host, 0, (kCallerSet + 1) * sizeof(unsigned));
+    if ((e = hipHostGetDevicePointer(&dev_view, host, 0)) != hipSuccess) return (int)e;
+    k.status_host = static_cast<volatile unsigned*>(host);
+    k.status_dev = static_cast<unsigned*>(dev_view);
     // 64 KB of dynamic LDS for KW = 2 is the default limit exactly; nothing to raise
     k.ready = true;
     g_device_ready[dev].store(true);
@@ -104,38 +158,98 @@ int asm_kernels(const AsmKernels** out) {
 
 // The same record if opencnn_init (or a launch) has set this device up already, else null: for
 // callers that must not load code objects or allocate.
-const AsmKernels* asm_kernels_if_ready() {
-  const AsmKernels* ak = nullptr;
+DeviceState* device_state_if_ready() {
+  DeviceState* ds = nullptr;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
   if (!g_device_ready[dev].load()) return nullptr;
-  return asm_kernels(&ak) == 0 ? ak : nullptr;
+  return device_state(&ds) == 0 ? ds : nullptr;
 }
 
-// The split-merge flags come in kSyncSets sets; every stream that launches gets a set of its own
-// for the life of the process, so launches that overlap in time (different streams) never share
-// flags, and launches on one stream are ordered anyway.  *sync stays null for a stream beyond
-// the kSyncSets-th: its launches then do without the split.
-int split_state(hipStream_t st, unsigned** sync) {
-  static hipStream_t owner[opencnn::kSyncSets];
-  static int used = 0;
-  static std::mutex mu;
-  *sync = nullptr;
-  const AsmKernels* ak = nullptr;
-  if (int e = asm_kernels(&ak)) return e;
-  std::lock_guard<std::mutex> lock(mu);
-  int set = -1;
-  for (int i = 0; i < used; ++i)
-    if (owner[i] == st) set = i;
-  if (set < 0 && used < opencnn::kSyncSets) {
-    owner[used] = st;
-    set = used++;
+// The split-merge flags come in kSyncSets sets of kSyncWords words.  Launches that may overlap in
+// time must not share one, launches that are ordered may:
+//   * a stream that launches directly holds one of the kEagerSets eager sets.  The library never
+//     asks a stream it does not launch on for its state (the handle may be stale: the stream may
+//     have been destroyed), so a set only changes hands on evidence of its own: once more streams
+//     have launched than there are sets ("pressure"), every launch is followed by an event of the
+//     set, and the set used longest ago whose event has completed goes to the stream that needs
+//     one.  opencnn_release_stream returns a set explicitly;
+//   * launches recorded during a stream capture may be replayed on any stream at any time, so
+//     they never share a set with direct launches: every (capture, stream) pair holds one of the
+//     kGraphSets graph sets for the life of the process.
+// *set stays -1 when none is free: that launch then does without the split.  A set that is handed
+// out is marked as having a call in flight until flag_set_launched().
+int flag_set_for(DeviceState* ds, hipStream_t st, int* set) {
+  *set = -1;
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  unsigned long long capture_id = 0;
+  if (st != nullptr) {  // the null stream cannot be captured
+    const hipError_t e = hipStreamGetCaptureInfo(st, &capture, &capture_id);
+    if (e != hipSuccess) return (int)e;
   }
-  if (set >= 0) *sync = ak->split_sync + (size_t)set * opencnn::kSyncWords;
+  std::lock_guard<std::mutex> lock(ds->flag_mu);
+  const bool graph = capture == hipStreamCaptureStatusActive;
+  const int first = graph ? opencnn::kEagerSets : 0;
+  const int last = graph ? opencnn::kSyncSets : opencnn::kEagerSets;
+  int found = -1, spare = -1;
+  for (int i = first; i < last; ++i) {
+    FlagSetOwner& o = ds->owners[i];
+    if (o.used && o.stream == st && (!graph || o.capture_id == capture_id)) found = i;
+    if (!o.used && spare < 0) spare = i;
+  }
+  if (found < 0) found = spare;
+  if (found < 0 && !graph) {
+    ds->pressure = true;
+    for (int i = 0; i < opencnn::kEagerSets; ++i) {
+      FlagSetOwner& o = ds->owners[i];
+      if (o.calls_in_flight != 0 || !o.idle_recorded) continue;
+      if (found >= 0 && o.last_use >= ds->owners[found].last_use) continue;
+      const hipError_t q = hipEventQuery(o.idle);
+      if (q == hipSuccess) found = i;
+      else (void)hipGetLastError();  // hipErrorNotReady: not the caller's error
+    }
+  }
+  if (found < 0) return 0;
+  FlagSetOwner& o = ds->owners[found];
+  if (!(o.used && o.stream == st)) o.idle_recorded = false;  // a new owner: nothing of it is recorded yet
+  o.used = true;
+  o.stream = st;
+  o.capture_id = graph ? capture_id : 0;
+  o.last_use = ++ds->clock;
+  ++o.calls_in_flight;
+  *set = found;
   return 0;
 }
 
-// Argument block of the assembly kernels (136 bytes, the layout gen_wino_f32_asm.py loads).
+// The call that took `set` has launched (or failed): under pressure, an event behind the launch
+// tells later calls when the set is idle.
+void flag_set_launched(DeviceState* ds, int set, hipStream_t st) {
+  if (set < 0 || set >= opencnn::kSyncSets) return;
+  std::lock_guard<std::mutex> lock(ds->flag_mu);
+  FlagSetOwner& o = ds->owners[set];
+  if (ds->pressure && set < opencnn::kEagerSets) {
+    if (o.idle == nullptr && hipEventCreateWithFlags(&o.idle, hipEventDisableTiming) != hipSuccess) o.idle = nullptr;
+    o.idle_recorded = o.idle != nullptr && hipEventRecord(o.idle, st) == hipSuccess;
+  }
+  --o.calls_in_flight;
+}
+
+// Gives the eager set of `st` back after waiting for the stream.
+int release_flag_set(DeviceState* ds, hipStream_t st) {
+  const hipError_t e = hipStreamSynchronize(st);
+  if (e != hipSuccess) return (int)e;
+  std::lock_guard<std::mutex> lock(ds->flag_mu);
+  for (int i = 0; i < opencnn::kEagerSets; ++i) {
+    FlagSetOwner& o = ds->owners[i];
+    if (o.used && o.stream == st && o.calls_in_flight == 0) {
+      o.used = false;
+      o.idle_recorded = false;
+    }
+  }
+  return 0;
+}
+
+// Argument block of the assembly kernels (152 bytes, the layout gen_wino_f32_asm.py loads).
 struct AsmKernArgs {
   const float* x;
   const float* usw;
@@ -148,8 +262,11 @@ struct AsmKernArgs {
   // (its sign selects the unit order) and the weighted length of a tile.
   int32_t c_real, k_real;
   long long* timeline;     // 64 entries per workgroup, or null
+  unsigned* status;        // status word of the flag set (a wave that gives up a wait stores 1)
+  uint32_t wait_polls;     // polls after which a wait for a flag gives up
+  uint32_t reserved;
 };
-static_assert(sizeof(AsmKernArgs) == 136, "kernel argument block");
+static_assert(sizeof(AsmKernArgs) == 152, "kernel argument block");
 
 // x / d == (x * m) >> s for 0 <= x < 2^31 (round-up method, 31-bit dividends).
 void magic_divisor(uint32_t d, uint32_t* m, uint32_t* s) {
@@ -160,9 +277,12 @@ void magic_divisor(uint32_t d, uint32_t* m, uint32_t* s) {
 }
 
 // Result of a HIP C++ kernel launch; remembers the kernel's name on success.
-int launched_hip(const char* name) {
+int launched_hip(const char* name, const dim3& grid) {
   const hipError_t e = hipGetLastError();
-  if (e == hipSuccess) t_last_kernel = name;
+  if (e == hipSuccess) {
+    t_last_kernel = name;
+    t_last_grid = (int)grid.x;
+  }
   return (int)e;
 }
 
@@ -208,13 +328,13 @@ int check_conv_shape(int in_n, int in_c, int in_h, int in_w, int filt_k) {
 }
 
 int launch_fx(const float* w, float* Ww, int filt_k, int filt_c, int filter_layout,
-              int ww_layout, hipStream_t st) {
+              int ww_layout, int precision, hipStream_t st) {
   REQUIRE(w != nullptr && Ww != nullptr);
   REQUIRE(filter_layout == OPENCNN_FILTER_CRSK || filter_layout == OPENCNN_FILTER_KCRS);
   REQUIRE(ww_layout == OPENCNN_WW_REFERENCE || ww_layout == OPENCNN_WW_MFMA);
   if (int e = check_filter_shape(filt_k, filt_c)) return e;
+  REQUIRE(precision == OPENCNN_F32 || precision == OPENCNN_F16 || precision == OPENCNN_BF16);
   const bool kcrs = filter_layout == OPENCNN_FILTER_KCRS;
-  const int precision = g_precision.load();
   if (ww_layout == OPENCNN_WW_MFMA && precision != OPENCNN_F32) {
     // padded to whole pairs of 32-wide filter groups and 16-channel chunks, zeros in the padding
     dim3 grid((unsigned)(padded_k_h16(filt_k) / 64), (unsigned)(padded_c_h16(filt_c) / 16)), block(256);
@@ -251,9 +371,9 @@ int launch_fx(const float* w, float* Ww, int filt_k, int filt_c, int filter_layo
 int launch_transpose(const float* src, float* dst, long long rows, long long cols, hipStream_t st) {
   REQUIRE(src != nullptr && dst != nullptr && src != dst);
   REQUIRE(rows > 0 && cols > 0 && rows * cols <= kMaxElems);
-  REQUIRE((rows + 63) / 64 <= 65535);  // gridDim.y
-  dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64)), block(256);
-  opencnn::transpose_2d<<<grid, block, 0, st>>>(src, dst, (int)rows, (int)cols);
+  const long long col_tiles = (cols + 63) / 64, row_tiles = (rows + 63) / 64;  // their product is below 2^31
+  dim3 grid((unsigned)(col_tiles * row_tiles)), block(256);
+  opencnn::transpose_2d<<<grid, block, 0, st>>>(src, dst, (int)rows, (int)cols, (int)col_tiles);
   return (int)hipGetLastError();
 }
 
@@ -286,7 +406,7 @@ int launch_h16(opencnn::ConvArgs a, int precision, hipStream_t st) {
     if (e != hipSuccess) return (int)e;
   }
   fn<<<grid, block, lds, st>>>(a);
-  return launched_hip("wino_h16_fused_lds");
+  return launched_hip("wino_h16_fused_lds", grid);
 }
 
 // A layer with fewer workgroup tiles than compute units would run one tile per workgroup, serially,
@@ -338,7 +458,7 @@ int asm_grid(const opencnn::ConvArgs& a, int kw, int chunks, CutTiles cut, int* 
   if (((long long)a.N * a.H * a.W * 4 + (long long)(a.W + 1) * a.N) * 4 > kMaxElems) return 0;
   int cus = 0;
   if (int e = compute_units(&cus)) return e;
-  const bool split = g_balance.load() != 0 && a.sync != nullptr;
+  const bool split = a.sync != nullptr;  // null: the balanced split is off, or no flag set was free
   if (a.nblocks < cus) {
     *grid = a.nblocks;  // one tile per workgroup
     if (split && cut == kCutPieces) *grid = a.nblocks * pieces_per_tile(a.nblocks, chunks, cus);
@@ -413,6 +533,8 @@ int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmLaunch& l, hipStream_
   ka.units_rem = (int32_t)(total % ranges);
   ka.usw_bytes = (int32_t)l.usw_bytes;
   ka.grid_per_xcd = grid % 8 == 0 ? grid / 8 : 0;  // 0: no XCD-aware block order
+  ka.status = a.status;
+  ka.wait_polls = a.spin_limit;
   ka.timeline = (size_t)grid * 64 * sizeof(long long) <= g_timeline_bytes.load() ? g_timeline.load() : nullptr;
   magic_divisor(chunk_divisor, &ka.m_chunks, &ka.s_chunks);
   if (l.natural_order) ka.s_chunks |= 64;
@@ -425,7 +547,10 @@ int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmLaunch& l, hipStream_
                    HIP_LAUNCH_PARAM_END};
   const hipError_t e = hipModuleLaunchKernel(l.fn, (unsigned)grid, 1, 1, 256, 1, 1, (unsigned)l.lds_bytes,
                                              st, nullptr, extra);
-  if (e == hipSuccess) t_last_kernel = l.name;
+  if (e == hipSuccess) {
+    t_last_kernel = l.name;
+    t_last_grid = grid;
+  }
   return (int)e;
 }
 
@@ -448,8 +573,7 @@ int pack_columns(opencnn::ConvArgs* a, int cw, int kblocks, int chunks, CutTiles
   const long long unpacked_tiles = ((long long)a->colgroups + cw - 1) / cw * kblocks;
   const long long packed_tiles = (packed_colgroups + cw - 1) / cw * kblocks;
   if (unpacked_tiles <= cus) {
-    const bool split = g_balance.load() != 0 && a->sync != nullptr;
-    if (!split) return 0;
+    if (a->sync == nullptr) return 0;  // no split
     // (cut into ranges, the layer's time follows its number of units: fewer tiles, fewer units)
     if (cut == kCutPieces &&
         pieces_per_tile((int)packed_tiles, chunks, cus) <= pieces_per_tile((int)unpacked_tiles, chunks, cus))
@@ -464,8 +588,8 @@ int pack_columns(opencnn::ConvArgs* a, int cw, int kblocks, int chunks, CutTiles
 
 int launch_asm(const opencnn::ConvArgs& a, int kw, int grid, bool ragged, bool packed, size_t lds_bytes,
                hipStream_t st) {
-  const AsmKernels* ak = nullptr;
-  if (int e = asm_kernels(&ak)) return e;
+  DeviceState* ak = nullptr;
+  if (int e = device_state(&ak)) return e;
   AsmLaunch l;
   if (packed) {
     l.fn = kw == 4 ? ak->kw4_packed : ak->kw2_packed;
@@ -518,8 +642,8 @@ int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* lau
   // here: these kernels' units are short, and a range that crosses a tile boundary pays two
   // output transforms and two hand-overs.)
   const bool cut_tiles = grid > a.nblocks;
-  const AsmKernels* ak = nullptr;
-  if (int e = asm_kernels(&ak)) return e;
+  DeviceState* ak = nullptr;
+  if (int e = device_state(&ak)) return e;
   AsmLaunch l;
   // the _ragged kernels mask batch elements, channels and filter rows that do not exist
   const bool ragged = a.N % 32 != 0 || a.C % 16 != 0 || a.K % 32 != 0;
@@ -567,20 +691,20 @@ int launch_hip(const opencnn::ConvArgs& a, int kw, bool ragged, bool allow_strea
       opencnn::wino_f32_fused<true><<<grid, block, 0, st>>>(a);
     else
       opencnn::wino_f32_fused<false><<<grid, block, 0, st>>>(a);
-    return launched_hip("wino_f32_fused");
+    return launched_hip("wino_f32_fused", grid);
   }
   if (ragged) {
     if (kw == 4)
       opencnn::wino_f32_fused_lds<4, false, true><<<grid, block, lds_bytes, st>>>(a);
     else
       opencnn::wino_f32_fused_lds<2, false, true><<<grid, block, lds_bytes, st>>>(a);
-    return launched_hip("wino_f32_fused_lds");
+    return launched_hip("wino_f32_fused_lds", grid);
   }
   // More tiles than CUs and not a whole number of rounds: one persistent workgroup per CU,
   // the chunk-units split evenly (every tile then has at most two contributors).
   int cus = 0;
   if (int e = compute_units(&cus)) return e;
-  const bool balanced = g_balance.load() != 0 && a.sync != nullptr && a.nblocks > cus && a.nblocks % cus != 0 &&
+  const bool balanced = a.sync != nullptr && a.nblocks > cus && a.nblocks % cus != 0 &&
                         cus % 8 == 0 && cus <= opencnn::kMaxBalancedBlocks &&
                         (long long)a.nblocks * (a.C / 8) <= kMaxElems;
   if (balanced) grid = dim3(cus);
@@ -602,13 +726,131 @@ int launch_hip(const opencnn::ConvArgs& a, int kw, bool ragged, bool allow_strea
     else
       opencnn::wino_f32_fused_lds<2, false><<<grid, block, lds_bytes, st>>>(a);
   }
-  return launched_hip(stream ? "wino_f32_stream" : "wino_f32_fused_lds");
+  return launched_hip(stream ? "wino_f32_stream" : "wino_f32_fused_lds", grid);
 }
 
+// ---- what the library knows about transformed filters it wrote
+// opencnn_filter_transform records, per buffer address, the form it wrote; the fused kernel refuses
+// a buffer whose record says another operand precision, layout or filter shape (it would read
+// 2-byte elements as floats, or the other way round, without any sign of it).  A buffer without a
+// record is taken as it is.
+struct WwRecord {
+  const void* ptr = nullptr;
+  int device = 0, precision = 0, layout = 0, filt_k = 0, filt_c = 0;
+  unsigned long long stamp = 0;
+};
+constexpr int kWwRecords = 64;
+WwRecord g_ww[kWwRecords];
+unsigned long long g_ww_clock = 0;
+std::mutex g_ww_mu;
+
+void remember_ww(const void* ptr, int precision, int layout, int filt_k, int filt_c) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return;
+  std::lock_guard<std::mutex> lock(g_ww_mu);
+  int slot = 0;
+  for (int i = 0; i < kWwRecords; ++i) {
+    if (g_ww[i].ptr == ptr && g_ww[i].device == dev) {
+      slot = i;
+      break;
+    }
+    if (g_ww[i].stamp < g_ww[slot].stamp) slot = i;  // else the record that is oldest
+  }
+  g_ww[slot].ptr = ptr;
+  g_ww[slot].device = dev;
+  g_ww[slot].precision = precision;
+  g_ww[slot].layout = layout;
+  g_ww[slot].filt_k = filt_k;
+  g_ww[slot].filt_c = filt_c;
+  g_ww[slot].stamp = ++g_ww_clock;
+}
+
+void forget_ww(const void* ptr) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return;
+  std::lock_guard<std::mutex> lock(g_ww_mu);
+  for (int i = 0; i < kWwRecords; ++i)
+    if (g_ww[i].ptr == ptr && g_ww[i].device == dev) g_ww[i] = WwRecord();
+}
+
+int check_ww(const void* ptr, int precision, int filt_k, int filt_c) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  std::lock_guard<std::mutex> lock(g_ww_mu);
+  for (int i = 0; i < kWwRecords; ++i) {
+    const WwRecord& r = g_ww[i];
+    if (r.ptr != ptr || r.device != dev) continue;
+    if (r.layout != OPENCNN_WW_MFMA) return fail("Ww holds the reference layout (OPENCNN_WW_REFERENCE), not what the fused kernel reads");
+    if (r.precision != precision) return fail("Ww was written under another operand precision");
+    if (r.filt_k != filt_k || r.filt_c != filt_c) return fail("Ww was written for another filter shape");
+    return 0;
+  }
+  return 0;
+}
+
+// Filter transform of a call, remembered per buffer.
+int transform_filter(const float* w, float* Ww, int filt_k, int filt_c, int filter_layout, int ww_layout,
+                     const CallSettings& c) {
+  if (int e = launch_fx(w, Ww, filt_k, filt_c, filter_layout, ww_layout, c.precision, c.stream)) return e;
+  remember_ww(Ww, ww_layout == OPENCNN_WW_MFMA ? c.precision : OPENCNN_F32, ww_layout, filt_k, filt_c);
+  return 0;
+}
+
+__global__ void zero_words(unsigned* p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+const char* const kGaveUp =
+    "an earlier launch gave up waiting for a partial tile (its output is invalid); the split-merge flags were cleared";
+
+// The flag set of this launch, and what an earlier launch may have left in its status word: a
+// wave that gave up a wait.  Then this call fails with hipErrorLaunchFailure and launches only
+// the kernel that clears the set (stream-ordered behind the launch that failed), so that the
+// call after it starts from clean flags.
+int prepare_split(DeviceState* ds, const CallSettings& c, opencnn::ConvArgs* a, int* taken) {
+  *taken = -1;
+  a->sync = nullptr;
+  a->status = ds->status_dev + kCallerSet;
+  a->spin_limit = g_wait_polls.load();
+  t_last_flag_set = -1;
+  if (!c.balance) return 0;
+  int set = -1;
+  if (c.caller_flags != nullptr) {
+    set = kCallerSet;
+    a->sync = c.caller_flags;
+  } else {
+    if (int e = flag_set_for(ds, c.stream, &set)) return e;
+    if (set < 0) return 0;
+    *taken = set;
+    a->sync = ds->split_sync + (size_t)set * opencnn::kSyncWords;
+  }
+  a->status = ds->status_dev + set;
+  if (ds->status_host[set] != 0) {
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (c.stream != nullptr) (void)hipStreamIsCapturing(c.stream, &capture);
+    if (capture == hipStreamCaptureStatusNone) {  // (a capture would record the repair instead of running it)
+      zero_words<<<(opencnn::kSyncWords + 255) / 256, 256, 0, c.stream>>>(a->sync, opencnn::kSyncWords);
+      (void)hipGetLastError();
+      ds->status_host[set] = 0;
+    }
+    flag_set_launched(ds, *taken, c.stream);
+    *taken = -1;
+    t_last_error = kGaveUp;
+    return (int)hipErrorLaunchFailure;
+  }
+  t_last_flag_set = set;
+  return 0;
+}
+
+int launch_on_flag_set(opencnn::ConvArgs& a, const CallSettings& c);
+
 int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c, int in_h,
-                int in_w, int filt_k, hipStream_t st) {
+                int in_w, int filt_k, const CallSettings& c) {
   REQUIRE(in != nullptr && Ww != nullptr && out != nullptr);
   if (int e = check_conv_shape(in_n, in_c, in_h, in_w, filt_k)) return e;
+  const int precision = c.precision;
+  if (int e = check_ww(Ww, precision, filt_k, in_c)) return e;
   opencnn::ConvArgs a;
   a.x = in;
   a.usw = Ww;
@@ -625,10 +867,22 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   a.colgroups = a.tiles_h * a.tiles_w * a.ngroups;
   a.kgroups = (filt_k + 31) / 32;
   a.nblocks = a.colblocks = 0;
-  if (int e = split_state(st, &a.sync)) return e;
-  const int precision = g_precision.load();
+  DeviceState* ds = nullptr;
+  if (int e = device_state(&ds)) return e;
+  int set = -1;
+  if (int e = prepare_split(ds, c, &a, &set)) return e;
+  const int rc = launch_on_flag_set(a, c);
+  flag_set_launched(ds, set, c.stream);
+  if (rc != 0) t_last_flag_set = -1;
+  return rc;
+}
+
+// The fused kernel of a call whose split-merge state is in place.
+int launch_on_flag_set(opencnn::ConvArgs& a, const CallSettings& c) {
+  const int in_n = a.N, in_c = a.C, filt_k = a.K, precision = c.precision;
+  hipStream_t st = c.stream;
   if (precision != OPENCNN_F32) {
-    const int v = g_variant.load();
+    const int v = c.variant;
     if (v == OPENCNN_KERNEL_ASM || v == OPENCNN_KERNEL_AUTO) {
       bool launched = false;
       if (int e = launch_h16_asm(a, precision, st, &launched)) return e;
@@ -639,7 +893,7 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   }
 
   const bool ragged = ragged_shape(in_n, in_c, filt_k);
-  const int variant = g_variant.load();
+  const int variant = c.variant;
   // kw = waves per workgroup that share one column tile (and split its input transform); the
   // workgroup's other dimension is 4 / kw column tiles.
   auto tile_with = [](opencnn::ConvArgs& a, int kw) {
@@ -679,6 +933,33 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   return launch_hip(a, kw, ragged, variant != OPENCNN_KERNEL_LDS, lds_bytes(kw), st);
 }
 
+bool valid_variant(int variant) {
+  return variant == OPENCNN_KERNEL_AUTO || variant == OPENCNN_KERNEL_REGISTER || variant == OPENCNN_KERNEL_LDS ||
+         variant == OPENCNN_KERNEL_ASM || variant == OPENCNN_KERNEL_HIP;
+}
+
+bool valid_precision(int precision) {
+  return precision == OPENCNN_F32 || precision == OPENCNN_F16 || precision == OPENCNN_BF16;
+}
+
+// The reference's dispatcher under the given settings.
+int forward_checked(float* k, int in_h, int in_w, float* w, int out_h, int out_w, int out_n, int out_c,
+                    float* C, float* Ww, int tiles_dim, int in_n, int tile_size, int in_c, int filt_k,
+                    int filt_c, int filt_h, int filt_w, int alpha, int m, const CallSettings& c) {
+  REQUIRE(k != nullptr && w != nullptr && C != nullptr && Ww != nullptr);
+  REQUIRE(filt_h == 3 && filt_w == 3);
+  REQUIRE(m == 2);
+  REQUIRE(alpha == 4 && tile_size == 4);
+  REQUIRE(in_h == in_w);  // the reference's masks and tiles_dim only model square images
+  REQUIRE(filt_c == in_c);
+  REQUIRE(out_h == in_h && out_w == in_w);  // pad 1, stride 1
+  REQUIRE(out_n == in_n && out_c == filt_k);
+  REQUIRE(tiles_dim == opencnn_tiles_dim(in_w));
+  if (int e = check_conv_shape(in_n, in_c, in_h, in_w, filt_k)) return e;
+  if (int e = transform_filter(w, Ww, filt_k, filt_c, OPENCNN_FILTER_CRSK, OPENCNN_WW_MFMA, c)) return e;
+  return launch_main(k, Ww, C, in_n, in_c, in_h, in_w, filt_k, c);
+}
+
 }  // namespace
 
 extern "C" {
@@ -686,6 +967,12 @@ extern "C" {
 const char* opencnn_last_error(void) { return t_last_error; }
 
 const char* opencnn_last_kernel(void) { return t_last_kernel; }
+
+int opencnn_last_launch(int* workgroups, int* flag_set) {
+  if (workgroups) *workgroups = t_last_grid;
+  if (flag_set) *flag_set = t_last_flag_set;
+  return 0;
+}
 
 int opencnn_init(void) {
   int dev = 0;
@@ -700,8 +987,8 @@ int opencnn_init(void) {
   }
   // load the assembly kernels now rather than inside the first launch (which may sit in a
   // stream capture or a timed region)
-  const AsmKernels* ak = nullptr;
-  return asm_kernels(&ak);
+  DeviceState* ds = nullptr;
+  return device_state(&ds);
 }
 
 int opencnn_tiles_dim(int in_w) {
@@ -716,15 +1003,15 @@ size_t opencnn_workspace_bytes(int filt_c, int filt_k) {
   return f32 > h16 ? f32 : h16;
 }
 
+size_t opencnn_split_flags_bytes(void) { return (size_t)opencnn::kSyncWords * sizeof(unsigned); }
+
 int opencnn_set_stream(void* stream) {
   g_stream.store(static_cast<hipStream_t>(stream));
   return 0;
 }
 
 int opencnn_set_kernel_variant(int variant) {
-  REQUIRE(variant == OPENCNN_KERNEL_AUTO || variant == OPENCNN_KERNEL_REGISTER ||
-          variant == OPENCNN_KERNEL_LDS || variant == OPENCNN_KERNEL_ASM ||
-          variant == OPENCNN_KERNEL_HIP);
+  REQUIRE(valid_variant(variant));
   g_variant.store(variant);
   return 0;
 }
@@ -745,7 +1032,7 @@ int opencnn_kcrs_to_crsk(const float* src, float* dst, int k, int c) {
 }
 
 int opencnn_set_operand_precision(int precision) {
-  REQUIRE(precision == OPENCNN_F32 || precision == OPENCNN_F16 || precision == OPENCNN_BF16);
+  REQUIRE(valid_precision(precision));
   g_precision.store(precision);
   return 0;
 }
@@ -763,14 +1050,50 @@ int opencnn_set_balanced_split(int enable) {
   return 0;
 }
 
+int opencnn_release_stream(void* stream) {
+  DeviceState* ds = device_state_if_ready();
+  if (ds == nullptr) return 0;
+  return release_flag_set(ds, static_cast<hipStream_t>(stream));
+}
+
+int opencnn_set_wait_limit(unsigned polls) {
+  g_wait_polls.store(polls == 0 ? kDefaultWaitPolls : polls);
+  return 0;
+}
+
+int opencnn_check_status(void) {
+  DeviceState* ds = device_state_if_ready();
+  if (ds == nullptr) return 0;  // nothing has been launched on this device
+  bool gave_up = false;
+  for (int set = 0; set <= kCallerSet; ++set) {
+    if (ds->status_host[set] == 0) continue;
+    gave_up = true;
+    if (set < kCallerSet) {
+      // the caller has synchronised: nothing that uses the flags is running
+      const hipError_t e = hipMemset(ds->split_sync + (size_t)set * opencnn::kSyncWords, 0,
+                                     opencnn::kSyncWords * sizeof(unsigned));
+      if (e != hipSuccess) return (int)e;
+    }
+    ds->status_host[set] = 0;
+  }
+  if (!gave_up) return 0;
+  t_last_error = kGaveUp;
+  return (int)hipErrorLaunchFailure;
+}
+
 int opencnn_filter_transform(const float* w, float* Ww, int filt_k, int filt_c,
                              int filter_layout, int ww_layout) {
-  return launch_fx(w, Ww, filt_k, filt_c, filter_layout, ww_layout, g_stream.load());
+  return transform_filter(w, Ww, filt_k, filt_c, filter_layout, ww_layout, process_settings());
+}
+
+int opencnn_forget_workspace(const void* Ww) {
+  forget_ww(Ww);
+  return 0;
 }
 
 int opencnn_conv_forward_pretransformed(const float* in, const float* Ww, float* out, int in_n,
                                         int in_c, int in_h, int in_w, int filt_k) {
-  return launch_main(in, Ww, out, in_n, in_c, in_h, in_w, filt_k, g_stream.load());
+  return launch_main(in, Ww, out, in_n, in_c, in_h, in_w, filt_k, process_settings());
 }
 
 int convolutionForward_32x64x8(float* k, int in_h, int in_w, float* w, int out_h, int out_w,
@@ -778,19 +1101,8 @@ int convolutionForward_32x64x8(float* k, int in_h, int in_w, float* w, int out_h
                                int tiles_dim, int in_n, int tile_size, int in_c, int filt_k,
                                int filt_c, int filt_h, int filt_w, int alpha, int m) {
   (void)n;  // out_c*out_n*out_h*out_w in the reference's bench; unused there too
-  REQUIRE(k != nullptr && w != nullptr && C != nullptr && Ww != nullptr);
-  REQUIRE(filt_h == 3 && filt_w == 3);
-  REQUIRE(m == 2);
-  REQUIRE(alpha == 4 && tile_size == 4);
-  REQUIRE(in_h == in_w);  // the reference's masks and tiles_dim only model square images
-  REQUIRE(filt_c == in_c);
-  REQUIRE(out_h == in_h && out_w == in_w);  // pad 1, stride 1
-  REQUIRE(out_n == in_n && out_c == filt_k);
-  REQUIRE(tiles_dim == opencnn_tiles_dim(in_w));
-  if (int e = check_conv_shape(in_n, in_c, in_h, in_w, filt_k)) return e;
-  hipStream_t st = g_stream.load();
-  if (int e = launch_fx(w, Ww, filt_k, filt_c, OPENCNN_FILTER_CRSK, OPENCNN_WW_MFMA, st)) return e;
-  return launch_main(k, Ww, C, in_n, in_c, in_h, in_w, filt_k, st);
+  return forward_checked(k, in_h, in_w, w, out_h, out_w, out_n, out_c, C, Ww, tiles_dim, in_n, tile_size,
+                         in_c, filt_k, filt_c, filt_h, filt_w, alpha, m, process_settings());
 }
 
 int convolutionForward(float* k, int in_h, int in_w, float* w, int out_h, int out_w, int out_n,
@@ -803,6 +1115,32 @@ int convolutionForward(float* k, int in_h, int in_w, float* w, int out_h, int ou
                                     filt_w, alpha, m);
 }
 
+int opencnn_conv_forward_desc(const opencnn_conv_desc* d) {
+  REQUIRE(d != nullptr);
+  REQUIRE(d->struct_size == sizeof(opencnn_conv_desc));
+  REQUIRE(d->in != nullptr && d->out != nullptr && d->Ww != nullptr);
+  REQUIRE(valid_variant(d->kernel_variant));
+  REQUIRE(valid_precision(d->operand_precision));
+  REQUIRE(d->filter_layout == OPENCNN_FILTER_CRSK || d->filter_layout == OPENCNN_FILTER_KCRS);
+  REQUIRE((d->split_flags == nullptr) == (d->split_flags_bytes == 0));
+  REQUIRE(d->split_flags == nullptr || d->split_flags_bytes >= opencnn_split_flags_bytes());
+  REQUIRE(d->split_flags == nullptr || reinterpret_cast<uintptr_t>(d->split_flags) % sizeof(unsigned) == 0);
+  if (int e = check_conv_shape(d->in_n, d->in_c, d->in_h, d->in_w, d->filt_k)) return e;
+  CallSettings c;
+  c.stream = static_cast<hipStream_t>(d->stream);
+  c.variant = d->kernel_variant;
+  c.precision = d->operand_precision;
+  c.balance = d->balanced_split != 0;
+  c.caller_flags = static_cast<unsigned*>(d->split_flags);
+  if (d->filter != nullptr) {
+    if (int e = transform_filter(d->filter, static_cast<float*>(d->Ww), d->filt_k, d->in_c, d->filter_layout,
+                                 OPENCNN_WW_MFMA, c))
+      return e;
+  }
+  return launch_main(d->in, static_cast<const float*>(d->Ww), d->out, d->in_n, d->in_c, d->in_h, d->in_w,
+                     d->filt_k, c);
+}
+
 int opencnn_conv_forward_static(const float* in, const float* w, float* out, int in_n, int in_c,
                                 int in_h, int in_w, int filt_k) {
   REQUIRE(in != nullptr && w != nullptr && out != nullptr);
@@ -810,14 +1148,14 @@ int opencnn_conv_forward_static(const float* in, const float* w, float* out, int
   if (int e = check_conv_shape(in_n, in_c, in_h, in_w, filt_k)) return e;
   if (opencnn_workspace_bytes(in_c, filt_k) > kScratchBytes)
     return fail("transformed filter exceeds the static workspace (opencnn_static_workspace_bytes)");
-  const AsmKernels* ak = asm_kernels_if_ready();
-  if (ak == nullptr) {
+  DeviceState* ds = device_state_if_ready();
+  if (ds == nullptr) {
     t_last_error = "opencnn_init() has not run on this device";
     return (int)hipErrorNotInitialized;
   }
-  hipStream_t st = g_stream.load();
-  if (int e = launch_fx(w, ak->scratch, filt_k, in_c, OPENCNN_FILTER_CRSK, OPENCNN_WW_MFMA, st)) return e;
-  return launch_main(in, ak->scratch, out, in_n, in_c, in_h, in_w, filt_k, st);
+  const CallSettings c = process_settings();
+  if (int e = transform_filter(w, ds->scratch, filt_k, in_c, OPENCNN_FILTER_CRSK, OPENCNN_WW_MFMA, c)) return e;
+  return launch_main(in, ds->scratch, out, in_n, in_c, in_h, in_w, filt_k, c);
 }
 
 size_t opencnn_static_workspace_bytes(void) { return kScratchBytes; }
@@ -828,7 +1166,8 @@ int opencnn_time_forward(const float* in, const float* w, float* out, float* Ww,
   REQUIRE(iters > 0 && warmup >= 0);
   REQUIRE(in != nullptr && w != nullptr && out != nullptr && Ww != nullptr);
   if (int e = check_conv_shape(in_n, in_c, in_h, in_w, filt_k)) return e;
-  hipStream_t st = g_stream.load();
+  const CallSettings c = process_settings();
+  hipStream_t st = c.stream;
   hipEvent_t ev[2];
   hipError_t he;
   if ((he = hipEventCreate(&ev[0])) != hipSuccess) return (int)he;
@@ -837,8 +1176,8 @@ int opencnn_time_forward(const float* in, const float* w, float* out, float* Ww,
     return (int)he;
   }
   int rc = 0;
-  auto fx = [&]() { return launch_fx(w, Ww, filt_k, in_c, OPENCNN_FILTER_CRSK, OPENCNN_WW_MFMA, st); };
-  auto maink = [&]() { return launch_main(in, Ww, out, in_n, in_c, in_h, in_w, filt_k, st); };
+  auto fx = [&]() { return transform_filter(w, Ww, filt_k, in_c, OPENCNN_FILTER_CRSK, OPENCNN_WW_MFMA, c); };
+  auto maink = [&]() { return launch_main(in, Ww, out, in_n, in_c, in_h, in_w, filt_k, c); };
   auto timed = [&](int mode, float* ms_out) {
     // mode 0: fx + main, 1: main only, 2: fx only
     for (int i = 0; i < warmup + iters && rc == 0; ++i) {

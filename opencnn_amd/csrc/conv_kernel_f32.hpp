@@ -50,7 +50,25 @@ struct ConvArgs {
                          // column block T % colblocks (LDS kernels): an XCD's contiguous
                          // range of tiles then needs one filter block's share of Ww, which
                          // fits its L2, instead of all of it
+  unsigned* status;      // status word of the flag set (host memory the GPU can write): a wave
+                         // that gives up waiting for a flag stores 1 there
+  unsigned spin_limit;   // polls after which a wait for a flag gives up
 };
+
+// Bounded wait for a split-merge flag.  A wave that gives up reports it in the launch's status
+// word and goes on with whatever the output tensor holds (the launch's result is wrong, but
+// every wave ends); the host finds the word at its next call.
+__device__ __forceinline__ void wait_for_flag(const ConvArgs& a, const unsigned* flag, int lane) {
+  unsigned spin = 0;
+  while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) == 0) {
+    if (++spin >= a.spin_limit) {
+      if (lane == 0) __hip_atomic_store(a.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      break;
+    }
+    __builtin_amdgcn_s_sleep(8);
+  }
+  asm volatile("" ::: "memory");  // the partial result is read after the flag, not before
+}
 
 // V = B^T d B, columns first then rows (src/convolutionForward_32x64x8.cu:59-80).
 __device__ __forceinline__ void input_transform(const float (&d)[16], float (&v)[16]) {
@@ -349,9 +367,11 @@ __global__ void __launch_bounds__(256) wino_f32_fused(ConvArgs a) {
 // wave that is already running its epilogue, never for one that has yet to be scheduled.
 constexpr int kMaxBalancedBlocks = 1024;
 // [set][boundary between workgroups b and b+1][wave] -> {ticket, flag}; zero between launches
-// (the second contributor clears its pair).  Launches that overlap in time must not share a
-// set: the host hands every stream its own (kSyncSets streams at most, see api.hip).
-constexpr int kSyncSets = 8;
+// (the second contributor clears its pair).  Launches that may overlap in time must not share a
+// set: the host hands one to every stream that launches and to every stream capture (api.hip).
+constexpr int kEagerSets = 32;  // streams that launch directly
+constexpr int kGraphSets = 16;  // launches recorded into HIP graphs
+constexpr int kSyncSets = kEagerSets + kGraphSets;
 constexpr int kSyncWords = kMaxBalancedBlocks * 4 * 2;
 static __device__ unsigned g_split_sync[kSyncSets * kSyncWords];
 
@@ -488,11 +508,7 @@ __global__ void __launch_bounds__(256) wino_f32_fused_lds(ConvArgs a) {
       if (lane == 0) __hip_atomic_store(sync + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     } else {
       // The first contributor holds ticket 0 and is in its epilogue; bounded wait all the same.
-      for (int spin = 0; spin < (1 << 22); ++spin) {
-        if (__hip_atomic_load(sync + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0) break;
-        __builtin_amdgcn_s_sleep(8);
-      }
-      asm volatile("" ::: "memory");  // the partial result is read after the flag, not before
+      wait_for_flag(a, sync + 1, lane);
       store_tile<kStoreMerge>(a, w, acc);
       if (lane == 0) {
         __hip_atomic_store(sync, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
@@ -761,11 +777,7 @@ __global__ void __launch_bounds__(256) wino_f32_stream(ConvArgs a) {
         } else {
           unsigned* flag = a.sync + (L * 4 + wave) * 2 + 1;
           // normally set long ago; bounded wait all the same (never hang the GPU on a bug)
-          for (int spin = 0; spin < (1 << 22); ++spin) {
-            if (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0) break;
-            __builtin_amdgcn_s_sleep(8);
-          }
-          asm volatile("" ::: "memory");  // the partial result is read after the flag, not before
+          wait_for_flag(a, flag, lane);
           store_tile<kStoreMerge>(a, w, acc);
           if (lane == 0) __hip_atomic_store(flag, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         }

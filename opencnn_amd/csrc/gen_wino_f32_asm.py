@@ -41,11 +41,17 @@ the last MFMA and v_accvgpr_read and between v_accvgpr_write and the next MFMA; 
 after v_readfirstlane before the SGPR is used; no vector instruction writes an SGPR while
 scalar loads are outstanding (v_readfirstlane next to s_load returned corrupted values).
 
-Kernel arguments (one 136-byte block, see AsmKernArgs in api.hip): four pointers (input CHWN,
-transformed filter in MFMA order, output KHWN, split-merge flags), 24 ints and the timeline
+Kernel arguments (one 152-byte block, see AsmKernArgs in api.hip): four pointers (input CHWN,
+transformed filter in MFMA order, output KHWN, split-merge flags), 24 ints, the timeline
 buffer (or null): 64 int64 per workgroup, [0] = number of stamps, [2..] = the 100 MHz realtime
 counter at kernel start, after the prologue and before / after every output transform, taken
-by the workgroup's first wave.
+by the workgroup's first wave; then the status word of the launch's flag set (host memory that
+the GPU can write) and the number of polls after which a wait for a flag gives up.
+
+A wait for a flag is bounded so that a bug or a workgroup that never becomes resident cannot
+hang the GPU.  A wave that gives up writes 1 to the status word and goes on with whatever the
+output tensor holds: the launch's result is wrong, every wave still ends, and the host finds
+the word at its next call (api.hip: the call fails and the flags are cleared).
 
 Usage: gen_wino_f32_asm.py > wino_f32_asm.s
 """
@@ -127,14 +133,15 @@ class Kernel:
         self.alloc_vgprs()
 
     def alloc_sgprs(self):
-        # s[0:1] kernel argument pointer, s2 workgroup id, s[8:15] the four pointers,
-        # s[16:39] the 24 ints, s[40:41] the timeline pointer, s42.. everything else
+        # s[0:1] kernel argument pointer, s2 workgroup id, s[4:5] the status word's address,
+        # s6 the poll limit of a flag wait, s[8:15] the four pointers, s[16:39] the 24 ints,
+        # s[40:41] the timeline pointer, s42.. everything else
         S = Alloc(42, 102)
         names = ["N", "H", "W", "Chunks", "TilesW", "Ngroups", "Colgroups", "Colblocks", "Q", "HWN4",
                  "UnitsQ", "UnitsRem", "UswBytes", "GridPerXcd", "Mch", "Sch", "Mcb", "Scb", "Mng",
                  "Sng", "Mtw", "Stw", "Creal", "Kreal", "Timeline", "TimelineHi"]
         self.S = {n: 16 + i for i, n in enumerate(names)}
-        self.S.update(X=8, U=10, Y=12, Sync=14)
+        self.S.update(X=8, U=10, Y=12, Sync=14, Status=4, SpinLimit=6)
         for n in ["L", "Kw", "Cw", "Wave", "Begin", "Nunits", "G", "Tp", "Cp", "Tq", "Cq", "Tm", "Cm",
                   "SegEnd", "Kind", "KgM", "KgQ", "ColStep", "RowStep", "Slab", "UoffM", "UoffQ",
                   "Dkb", "Dlive", "Dng", "Dty", "Dtx", "RowOk", "Spin", "KwSpw"]:
@@ -761,11 +768,13 @@ class Kernel:
         self.e("s_mov_b64 exec, -1")
 
     def wait_flag(self):
-        """Until the workgroup behind this one has published its part of the tile (bounded)."""
+        """Until the workgroup behind this one has published its part of the tile.  Bounded by
+        SpinLimit polls: a wave that gives up reports it in the status word (out of line) and
+        goes on, so that every wave ends whatever happens to the publisher."""
         t = self.t
         self.flag_address(False)
         self.e(f"s_mov_b32 {self.sr('Spin')}, 0")
-        poll, got = self.newlabel("poll"), self.newlabel("got")
+        poll, got, giveup = self.newlabel("poll"), self.newlabel("got"), self.newlabel("giveup")
         self.label(poll)
         self.e(f"global_load_dword {self.vr('Tmp')}, {self.vr('Zero')}, {s(self.S['Fl'], 2)} sc0 sc1")
         self.e("s_waitcnt vmcnt(0)")
@@ -774,11 +783,19 @@ class Kernel:
         self.e(f"s_cmp_lg_u32 {t(0)}, 0")
         self.e(f"s_cbranch_scc1 {got}")
         self.e(f"s_add_u32 {self.sr('Spin')}, {self.sr('Spin')}, 1")
-        self.e(f"s_cmp_lt_u32 {self.sr('Spin')}, 0x100000")
-        self.e(f"s_cbranch_scc0 {got}")  # never hang the GPU on a bug: give up and produce a wrong tile
+        self.e(f"s_cmp_lt_u32 {self.sr('Spin')}, {self.sr('SpinLimit')}")
+        self.e(f"s_cbranch_scc0 {giveup}")
         self.e("s_sleep 8")
         self.e(f"s_branch {poll}")
         self.label(got)
+        main, self.lines = self.lines, []
+        self.label(giveup)
+        self.e("s_mov_b64 exec, 1")
+        self.e(f"global_store_dword {self.vr('Zero')}, {self.vr('One')}, {s(self.S['Status'], 2)} sc0 sc1")
+        self.e("s_mov_b64 exec, -1")
+        self.e(f"s_branch {got}")
+        self.outofline.extend(self.lines)
+        self.lines = main
 
     def late_merge_registers(self):
         """64 registers for the partial tile of a late merge: the filter operands."""
@@ -883,6 +900,8 @@ class Kernel:
         e(f"s_load_dwordx16 {s(16, 16)}, s[0:1], 0x20")
         e(f"s_load_dwordx8 {s(32, 8)}, s[0:1], 0x60")
         e(f"s_load_dwordx2 {s(40, 2)}, s[0:1], 0x80")
+        e(f"s_load_dwordx2 {s(S['Status'], 2)}, s[0:1], 0x88")
+        e(f"s_load_dword {self.sr('SpinLimit')}, s[0:1], 0x90")
         e(f"v_and_b32 {self.vr('Tmp', 1)}, 0x3ff, v0")
         e(f"v_lshrrev_b32 {self.vr('Tmp')}, 6, {self.vr('Tmp', 1)}")
         e(f"v_and_b32 {self.vr('Lane')}, 63, {self.vr('Tmp', 1)}")
@@ -1064,7 +1083,7 @@ class Kernel:
 \t.amdhsa_kernel {n}
 \t\t.amdhsa_group_segment_fixed_size 0
 \t\t.amdhsa_private_segment_fixed_size 0
-\t\t.amdhsa_kernarg_size 136
+\t\t.amdhsa_kernarg_size 152
 \t\t.amdhsa_user_sgpr_count 2
 \t\t.amdhsa_user_sgpr_kernarg_segment_ptr 1
 \t\t.amdhsa_system_sgpr_workgroup_id_x 1
@@ -1092,13 +1111,23 @@ class Kernel:
       - .address_space:  global
         .offset:         128
         .size:           8
-        .value_kind:     global_buffer"""
+        .value_kind:     global_buffer
+      - .address_space:  global
+        .offset:         136
+        .size:           8
+        .value_kind:     global_buffer
+      - .offset:         144
+        .size:           4
+        .value_kind:     by_value
+      - .offset:         148
+        .size:           4
+        .value_kind:     by_value"""
         return f"""  - .agpr_count:     256
     .args:
 {args}
     .group_segment_fixed_size: 0
     .kernarg_segment_align: 8
-    .kernarg_segment_size: 136
+    .kernarg_segment_size: 152
     .max_flat_workgroup_size: 256
     .name:           {self.name}
     .private_segment_fixed_size: 0

@@ -12,11 +12,14 @@
 
 namespace opencnn {
 
+// One-dimensional grid over the 64x64 tiles, a row of tiles after the other (gridDim.x takes
+// 2^31 - 1 blocks, so neither side of the matrix is limited by the 65535 of the other dimensions).
 __global__ void __launch_bounds__(256) transpose_2d(const float* __restrict__ src, float* __restrict__ dst,
-                                                    int rows, int cols) {
+                                                    int rows, int cols, int col_tiles) {
   __shared__ float tile[64][65];
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 x 4 threads
-  const int c0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
+  const int row_tile = blockIdx.x / col_tiles;
+  const int c0 = (blockIdx.x - row_tile * col_tiles) * 64, r0 = row_tile * 64;
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
     const int r = r0 + ty + 4 * i, c = c0 + tx;

@@ -159,6 +159,7 @@ int main(int argc, char** argv) {
   std::vector<double> want(n_out);
   HIP_CALL(hipMemcpy(got.data(), out_data, n_out * sizeof(float), hipMemcpyDeviceToHost));
   HIP_CALL(hipMemcpy(want.data(), ref_data, n_out * sizeof(double), hipMemcpyDeviceToHost));
+  OPENCNN_CALL(opencnn_check_status());  // every launch handed its partial tiles over
   double max_error = 0.0, num = 0.0, den = 0.0;
   long bad = 0;
   for (size_t i = 0; i < n_out; ++i) {

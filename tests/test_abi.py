@@ -72,6 +72,38 @@ def test_filter_transform_rejects_bad_arguments(ocn):
     assert f(0, 0x1000, 64, 8, 0, 0) == 1
 
 
+def test_descriptor_is_validated_before_any_launch(ocn):
+    d = ocn.ConvDesc()
+    call = lambda: ocn.lib().opencnn_conv_forward_desc(ctypes.byref(d))
+    assert ocn.lib().opencnn_conv_forward_desc(None) == 1
+    assert call() == 1  # struct_size 0
+    d.struct_size = ctypes.sizeof(ocn.ConvDesc)
+    assert ctypes.sizeof(ocn.ConvDesc) == 104  # the layout of opencnn_conv_desc on LP64
+    assert call() == 1  # null tensors
+    d.in_ = d.out = d.Ww = d.filter = 0x1000
+    d.in_n, d.in_c, d.in_h, d.in_w, d.filt_k = 32, 8, 8, 8, 64
+    for field, bad in (("operand_precision", 3), ("kernel_variant", 5), ("filter_layout", 2), ("in_c", 0),
+                       ("split_flags_bytes", 4096)):
+        good = getattr(d, field)
+        setattr(d, field, bad)
+        assert call() == 1, field
+        assert ocn.lib().opencnn_last_error() != b""
+        setattr(d, field, good)
+    d.split_flags, d.split_flags_bytes = 0x2000, ocn.split_flags_bytes() - 4
+    assert call() == 1  # flag storage too small
+    d.split_flags, d.split_flags_bytes = 0x2002, ocn.split_flags_bytes()
+    assert call() == 1  # misaligned
+    assert ocn.split_flags_bytes() == 32768
+
+
+def test_status_query_without_a_launch(ocn):
+    # nothing has run on any device: nothing to report, and nothing that needs a GPU
+    assert ocn.lib().opencnn_check_status() == 0
+    assert ocn.lib().opencnn_set_wait_limit(0) == 0
+    assert ocn.lib().opencnn_forget_workspace(0x1000) == 0
+    assert ocn.last_launch() == (0, -1)
+
+
 def test_synth_layouts_agree(ocn):
     N, C, H, W, K = 32, 8, 5, 6, 64
     chwn = ocn.synth_input(N, C, H, W, seed=0x0C99)

@@ -73,6 +73,50 @@ def test_kernel_text_invariants(gen, kw, ragged, packed):
         assert target in labels
 
 
+def check_bounded_waits(k, text):
+    """Every wait for a flag (merge in front of a segment, two merges inside an output transform)
+    is bounded by the poll limit of the argument block, and the wave that gives up stores to the
+    status word before it goes on: no silent wrong tile, no endless loop."""
+    polls = re.findall(r"^(\.L\w+_poll_\d+):", text, re.M)
+    assert len(polls) == 3
+    limit, status = f"s{k.S['SpinLimit']}", f"s[{k.S['Status']}:{k.S['Status'] + 1}]"
+    assert f"s_load_dwordx2 {status}, s[0:1], 0x88" in text
+    assert f"s_load_dword {limit}, s[0:1], 0x90" in text
+    assert "0x100000" not in text  # no compiled-in limit left
+    lines = text.splitlines()
+    for poll in polls:
+        i = lines.index(poll + ":")
+        loop = lines[i:i + 14]
+        back = [j for j, l in enumerate(loop) if l.strip() == f"s_branch {poll}"]
+        assert back, "poll loop without its backward branch"
+        loop = loop[:back[0] + 1]
+        # the only ways out: the flag is there, or the limit is reached
+        exits = [l.split()[-1] for l in loop if "s_cbranch" in l]
+        assert len(exits) == 2
+        got, giveup = exits
+        assert "_got_" in got and "_giveup_" in giveup
+        cmp_limit = [j for j, l in enumerate(loop) if l.strip().startswith("s_cmp_lt_u32") and l.strip().endswith(limit)]
+        assert cmp_limit and "s_cbranch_scc0 " + giveup in loop[cmp_limit[0] + 1]
+        j = lines.index(giveup + ":")
+        block = [l.strip() for l in lines[j + 1:j + 5]]
+        assert block[0] == "s_mov_b64 exec, 1"
+        assert re.fullmatch(r"global_store_dword v\d+, v\d+, " + re.escape(status) + " sc0 sc1", block[1])
+        assert block[1].split()[2].rstrip(",") == f"v{k.V['One']}"
+        assert block[2] == "s_mov_b64 exec, -1" and block[3] == f"s_branch {got}"
+    # the status word's registers are written by the argument load only
+    for reg in (k.S["Status"], k.S["Status"] + 1, k.S["SpinLimit"]):
+        writers = re.findall(rf"^\s*([sv]_\w+) s{reg}\b", text, re.M)
+        assert writers in (["s_load_dword"], []), writers
+
+
+@pytest.mark.parametrize("ragged,packed", VARIANTS)
+@pytest.mark.parametrize("kw", [2, 4])
+def test_flag_waits_are_bounded_and_report(gen, kw, ragged, packed):
+    k = gen.Kernel(kw, ragged, packed)
+    k.body()
+    check_bounded_waits(k, "\n".join(k.lines))
+
+
 @pytest.mark.skipif(not os.path.exists(CLANG), reason="ROCm LLVM assembler not installed")
 def test_output_assembles_for_gfx950(tmp_path):
     src = tmp_path / "k.s"
@@ -148,6 +192,14 @@ def test_h16_kernel_text_invariants(gen_h16, bf16, ragged, packed):
         assert target in labels
     # LDS: two 16 KB buffers; every access stays below 32 KB for the largest lane offsets
     assert max(int(n) for n in re.findall(r"offset1:(\d+)", text)) * 256 + 0x4000 + 0x80 + 636 < 32768
+
+
+@pytest.mark.parametrize("ragged,packed", VARIANTS)
+@pytest.mark.parametrize("bf16", [False, True])
+def test_h16_flag_waits_are_bounded_and_report(gen_h16, bf16, ragged, packed):
+    k = gen_h16.KernelH16(bf16, ragged, packed)
+    k.body()
+    check_bounded_waits(k, "\n".join(k.lines))
 
 
 @pytest.mark.skipif(not os.path.exists(CLANG), reason="ROCm LLVM assembler not installed")

@@ -780,8 +780,8 @@ def test_non_default_stream(ocn, oracle, torch_gpu):
 def test_layers_on_different_streams_may_overlap(ocn, oracle, torch_gpu):
     # two layers whose tiles are cut between workgroups (784 and 800 tiles on 256 CUs), launched
     # back to back on two streams without synchronisation in between, so that they may run at the
-    # same time: every stream has split-merge flags of its own, the results are the serial ones.
-    # Ten streams in all: more than the library has flag sets for (the extra ones run unsplit).
+    # same time: every stream has split-merge flags of its own, the results are the serial ones,
+    # bit for bit.  Ten streams in all.
     print("overlapping streams", flush=True)
     torch = torch_gpu
     shapes = [(64, 32, 56, 56, 64), (64, 32, 40, 40, 128)]
@@ -801,12 +801,10 @@ def test_layers_on_different_streams_may_overlap(ocn, oracle, torch_gpu):
             for i, r in enumerate(runners):
                 ocn.set_stream(streams[(2 * rep + i) % len(streams)])
                 ocn.conv_forward_pretransformed(r.xd, r.ws, r.yd, r.N, r.C, r.H, r.W, r.K)
+                assert ocn.last_launch()[1] >= 0, "launched without the split"
             torch.cuda.synchronize()
             for r, y in zip(runners, want):
-                # not bit for bit: a stream without flags of its own runs the unsplit launch, which
-                # associates the channel sum differently; a lost or foreign partial tile is far off
-                rel, _, _ = oracle.compare(r.result(), y)
-                assert rel <= 1e-6, f"rep {rep}: rel-L2 against the serial result {rel:.3e}"
+                assert np.array_equal(r.result(), y), f"rep {rep}"
     finally:
         ocn.set_stream(None)
 
@@ -892,8 +890,14 @@ def test_call_replays_from_a_captured_graph(ocn, oracle, torch_gpu, N, C, H, K):
         with torch.cuda.stream(s):
             launch()
             s.synchronize()
+            eager = (ocn.last_kernel(), ocn.last_launch()[0])
             with torch.cuda.graph(g, stream=s):
                 launch()
+        # the captured launch is the eager one (same kernel, same grid) on a flag set of its own
+        assert (ocn.last_kernel(), ocn.last_launch()[0]) == eager
+        assert ocn.last_launch()[1] >= 32, "the captured launch shares flags with direct launches"
+        if (N, C, H, K) != (32, 8, 8, 64):
+            assert ocn.last_kernel().startswith("wino_f32_asm") and ocn.last_launch()[0] > 64
         for rep in range(3):
             x2, w2 = ocn.synth_input(N, C, H, H, seed=100 + rep), ocn.synth_filter(K, C, seed=200 + rep)
             r.xd.copy_(torch.from_numpy(x2).to(r.xd.device))
