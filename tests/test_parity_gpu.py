@@ -583,7 +583,8 @@ def test_padded_channels_do_not_leak_non_finite_values(ocn, oracle, torch_gpu, p
 
 # ---------------------------------------------------------------- layout shims
 
-@pytest.mark.parametrize("N,C,H,W,K", [(32, 8, 8, 8, 64), (64, 64, 56, 56, 64), (96, 1030, 5, 3, 33), (1, 1, 1, 1, 1)])
+@pytest.mark.parametrize("N,C,H,W,K", [(32, 8, 8, 8, 64), (64, 64, 56, 56, 64), (96, 1030, 5, 3, 33), (1, 1, 1, 1, 1),
+                                       (2, 3, 224, 224, 128)])  # K*H*W beyond 65535 rows of 64
 def test_layout_shims_are_exact_permutations(ocn, torch_gpu, N, C, H, W, K):
     # the reference's data_cpy transposes (src/openCNN_winograd.cu:147-153,230,235): bit-exact,
     # checked against numpy; C = 1030 is beyond data_cpy's C <= 1024 launch limit
