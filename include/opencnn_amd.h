@@ -326,6 +326,18 @@ int opencnn_time_forward(const float *in, const float *w, float *out, float *Ww,
                          int iters, float *ms_total, float *ms_main, float *ms_fx);
 
 /*
+ * Bench support without a counterpart in the reference: the order in which the assembly kernels
+ * walk through the tiles of the image, which decides how much of a tile's input patch is found in
+ * the L2 of its XCD because a neighbouring tile has just read it.  Results do not depend on it.
+ * Bits: 1 = neighbouring column tiles are neighbouring spatial tiles (else: the same spatial tile
+ * of the next 32 batch elements), 2 = spatial tiles numbered in zigzag strips of two tile rows
+ * (else row by row), 4 = fp16 / bf16 kernels: the tiles that an XCD's workgroups start with lie
+ * together in the image, the tiles they go on with beside them.  Default 7; 0 is the order of
+ * the first version of the kernels, kept for measurements (profiles/).
+ */
+int opencnn_set_tile_order(int bits);
+
+/*
  * Bench support without a counterpart in the reference: a timeline of the assembly kernels.
  * While a buffer is set, the first wave of workgroup L of every later launch of those kernels
  * writes into device_buffer[L*64 ...]: [0] the number of stamps, [2], [3], ... the GPU's

@@ -77,6 +77,7 @@ EXPORTED_SYMBOLS = {
     "opencnn_check_status": (_c_int, []),
     "opencnn_release_stream": (_c_int, [_c_void_p]),
     "opencnn_set_wait_limit": (_c_int, [ctypes.c_uint]),
+    "opencnn_set_tile_order": (_c_int, [_c_int]),
     "opencnn_forget_workspace": (_c_int, [_c_void_p]),
     "opencnn_conv_forward_desc": (_c_int, [_c_void_p]),
     "opencnn_split_flags_bytes": (ctypes.c_size_t, []),
@@ -200,6 +201,11 @@ def release_stream(stream) -> None:
     """Wait for `stream` and give its set of split-merge flags back."""
     handle = 0 if stream is None else getattr(stream, "cuda_stream", stream)
     _check("opencnn_release_stream", lib().opencnn_release_stream(handle))
+
+
+def set_tile_order(bits: int) -> None:
+    """Order of the tiles in the image (bits 1, 2, 4 of opencnn_set_tile_order; default 7)."""
+    _check("opencnn_set_tile_order", lib().opencnn_set_tile_order(bits))
 
 
 def set_wait_limit(polls: int) -> None:

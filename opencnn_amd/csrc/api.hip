@@ -28,6 +28,9 @@ std::atomic<bool> g_device_ready[64];  // set-up of device_state() done on that 
 // Polls after which a kernel's wait for a split-merge flag gives up (about a second).
 constexpr unsigned kDefaultWaitPolls = 1u << 20;
 std::atomic<unsigned> g_wait_polls{kDefaultWaitPolls};
+// Order of the tiles in the image (bits: 1 spatial tile fastest, 2 strips of two tile rows, 4 places
+// by starting time), see AsmLaunch; all on.  opencnn_set_tile_order is bench support.
+std::atomic<int> g_tile_order{7};
 
 // The settings of one call: what the opencnn_set_* calls select for the entry points that take no
 // descriptor, or the fields of an opencnn_conv_desc.
@@ -249,7 +252,7 @@ int release_flag_set(DeviceState* ds, hipStream_t st) {
   return 0;
 }
 
-// Argument block of the assembly kernels (152 bytes, the layout gen_wino_f32_asm.py loads).
+// Argument block of the assembly kernels (168 bytes, the layout gen_wino_f32_asm.py loads).
 struct AsmKernArgs {
   const float* x;
   const float* usw;
@@ -264,9 +267,13 @@ struct AsmKernArgs {
   long long* timeline;     // 64 entries per workgroup, or null
   unsigned* status;        // status word of the flag set (a wave that gives up a wait stores 1)
   uint32_t wait_polls;     // polls after which a wait for a flag gives up
+  // fp16 / bf16 kernels: the places of a line's tiles (KernelH16.place): magic number of the
+  // tiles on the line (bit 6 of the shift switches the places on), ranges and tiles on the line
+  uint32_t m_place, s_place;
+  int32_t place_ranges, place_tiles;
   uint32_t reserved;
 };
-static_assert(sizeof(AsmKernArgs) == 152, "kernel argument block");
+static_assert(sizeof(AsmKernArgs) == 168, "kernel argument block");
 
 // x / d == (x * m) >> s for 0 <= x < 2^31 (round-up method, 31-bit dividends).
 void magic_divisor(uint32_t d, uint32_t* m, uint32_t* s) {
@@ -494,6 +501,19 @@ struct AsmLaunch {
   // fp16 / bf16 kernels: ranges shorter than a tile, walked in the natural chunk order (flagged in
   // bit 6 of the units' magic shift, which the kernel's 64-bit shifts ignore)
   bool natural_order = false;
+  // Order of the column tiles on their line: image group fastest (the same spatial tile of the next
+  // 32 batch elements follows), or spatial tile fastest (neighbours on the line are neighbours in
+  // the image, image group after image group).
+  // Measured on the fp16 benchmark layer (N=128 C=K=256 14x14), fabric reads per launch: image
+  // group fastest 124.6 MB, spatial tile fastest 93.2 MB (-3 % time); fp32 N=64 C=K=64 56x56
+  // 155.5 -> 137.4 MB.
+  bool spatial_fastest = g_tile_order.load() & 1;
+  // Spatial tiles numbered in strips of two tile rows, zigzag, instead of row by row (fp32
+  // N=64 C=K=64 56x56: 137.4 -> 129.3 MB, -0.5 % time).
+  bool strips = g_tile_order.load() & 2;
+  // fp16 / bf16 kernels: the tiles in work from the start get the first places of an XCD's window
+  // (KernelH16.place; 93.3 -> 82.4 MB on the fp16 benchmark layer).
+  bool tile_places = g_tile_order.load() & 4;
 };
 
 int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmLaunch& l, hipStream_t st) {
@@ -529,6 +549,16 @@ int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmLaunch& l, hipStream_
     ka.k_real = (int32_t)vt;
     chunk_divisor = (uint32_t)vt;
   }
+  if (l.filters >= 0) {
+    // the line of tiles the ranges are cut from, before its weights: one per filter block, or one
+    const long long line_tiles = l.lockstep_log2 >= 0 ? a.nblocks >> l.lockstep_log2 : a.nblocks;
+    ka.place_tiles = (int32_t)line_tiles;
+    ka.place_ranges = ranges;
+    magic_divisor((uint32_t)line_tiles, &ka.m_place, &ka.s_place);
+    if (l.tile_places && !l.packed && !l.natural_order && ranges % 8 == 0 && ranges <= line_tiles &&
+        line_tiles * ranges + ranges <= kMaxElems && line_tiles * 8 <= kMaxElems)
+      ka.s_place |= 64;
+  }
   ka.units_q = (int32_t)(total / ranges);
   ka.units_rem = (int32_t)(total % ranges);
   ka.usw_bytes = (int32_t)l.usw_bytes;
@@ -540,8 +570,15 @@ int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmLaunch& l, hipStream_
   if (l.natural_order) ka.s_chunks |= 64;
   magic_divisor((uint32_t)l.tile_split, &ka.m_colblocks, &ka.s_colblocks);
   if (l.lockstep_log2 >= 0) ka.s_colblocks = (uint32_t)l.lockstep_log2;
-  magic_divisor((uint32_t)(l.packed ? a.N : a.ngroups), &ka.m_ngroups, &ka.s_ngroups);
+  if (!l.packed && l.spatial_fastest) {
+    ka.ngroups = a.tiles_h * a.tiles_w;
+    magic_divisor((uint32_t)ka.ngroups, &ka.m_ngroups, &ka.s_ngroups);
+    ka.s_ngroups |= 64;
+  } else {
+    magic_divisor((uint32_t)(l.packed ? a.N : a.ngroups), &ka.m_ngroups, &ka.s_ngroups);
+  }
   magic_divisor((uint32_t)a.tiles_w, &ka.m_tiles_w, &ka.s_tiles_w);
+  if (!l.packed && l.strips) ka.s_tiles_w |= 64;
   size_t ka_size = sizeof(ka);
   void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &ka, HIP_LAUNCH_PARAM_BUFFER_SIZE, &ka_size,
                    HIP_LAUNCH_PARAM_END};
@@ -1054,6 +1091,12 @@ int opencnn_release_stream(void* stream) {
   DeviceState* ds = device_state_if_ready();
   if (ds == nullptr) return 0;
   return release_flag_set(ds, static_cast<hipStream_t>(stream));
+}
+
+int opencnn_set_tile_order(int bits) {
+  REQUIRE(bits >= 0 && bits <= 7);
+  g_tile_order.store(bits);
+  return 0;
 }
 
 int opencnn_set_wait_limit(unsigned polls) {

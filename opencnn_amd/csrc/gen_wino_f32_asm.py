@@ -41,7 +41,7 @@ the last MFMA and v_accvgpr_read and between v_accvgpr_write and the next MFMA; 
 after v_readfirstlane before the SGPR is used; no vector instruction writes an SGPR while
 scalar loads are outstanding (v_readfirstlane next to s_load returned corrupted values).
 
-Kernel arguments (one 152-byte block, see AsmKernArgs in api.hip): four pointers (input CHWN,
+Kernel arguments (one 168-byte block, see AsmKernArgs in api.hip): four pointers (input CHWN,
 transformed filter in MFMA order, output KHWN, split-merge flags), 24 ints, the timeline
 buffer (or null): 64 int64 per workgroup, [0] = number of stamps, [2..] = the 100 MHz realtime
 counter at kernel start, after the prologue and before / after every output transform, taken
@@ -51,7 +51,8 @@ the GPU can write) and the number of polls after which a wait for a flag gives u
 A wait for a flag is bounded so that a bug or a workgroup that never becomes resident cannot
 hang the GPU.  A wave that gives up writes 1 to the status word and goes on with whatever the
 output tensor holds: the launch's result is wrong, every wave still ends, and the host finds
-the word at its next call (api.hip: the call fails and the flags are cleared).
+the word at its next call (api.hip: the call fails and the flags are cleared).  The last four
+ints (the places of the tiles of a line in the image) are read by the fp16 / bf16 kernels only.
 
 Usage: gen_wino_f32_asm.py > wino_f32_asm.s
 """
@@ -216,12 +217,41 @@ class Kernel:
             self.e(f"s_mov_b32 {self.sr('Dng')}, 0")
             self.e(f"s_mov_b32 {self.sr('Dtx')}, 0")
             return
-        self.div(t(2), t(0), self.sr("Mng"), self.sr("Sng"))  # spatial tile
+        # Column tile -> (spatial tile, image group).  The argument slot Ngroups holds the divisor:
+        # the image groups when they are the fast index of the line of column tiles, or, with bit 6
+        # of the magic shift set (64-bit shifts ignore it), the spatial tiles when those are.
+        self.div(t(2), t(0), self.sr("Mng"), self.sr("Sng"))
         self.e(f"s_mul_i32 {t(3)}, {t(2)}, {self.sr('Ngroups')}")
-        self.e(f"s_sub_u32 {self.sr('Dng')}, {t(0)}, {t(3)}")
+        self.e(f"s_sub_u32 {t(3)}, {t(0)}, {t(3)}")
+        self.e(f"s_bitcmp1_b32 {self.sr('Sng')}, 6")
+        self.e(f"s_cselect_b32 {self.sr('Dng')}, {t(2)}, {t(3)}")
+        self.e(f"s_cselect_b32 {t(2)}, {t(3)}, {t(2)}")  # spatial tile
         self.div(self.sr("Dty"), t(2), self.sr("Mtw"), self.sr("Stw"))
         self.e(f"s_mul_i32 {t(3)}, {self.sr('Dty')}, {self.sr('TilesW')}")
         self.e(f"s_sub_u32 {self.sr('Dtx')}, {t(2)}, {t(3)}")
+        # With bit 6 of the magic shift Stw set, the spatial tiles are numbered in strips of two
+        # tile rows, zigzag: neighbours on the line are neighbours in the image in both directions
+        # (tile i+1 below or beside tile i, tile i+2 beside it).  (row r0, column c0) of the
+        # row-major reading -> strip r0 / 2, position (r0 % 2) * TilesW + c0 inside it; a last
+        # strip of one row keeps its row-major order.
+        # (No branch: in the fp32 kernels this code is dealt out over the gaps between MFMAs.)
+        self.e(f"s_add_u32 {t(3)}, {self.sr('H')}, 1")
+        self.e(f"s_lshr_b32 {t(3)}, {t(3)}, 1")                    # tile rows
+        self.e(f"s_or_b32 {t(4)}, {self.sr('Dty')}, 1")
+        self.e(f"s_cmp_lt_u32 {t(4)}, {t(3)}")                      # the strip has two rows
+        self.e(f"s_cselect_b32 {t(5)}, 1, 0")
+        self.e(f"s_bitcmp1_b32 {self.sr('Stw')}, 6")
+        self.e(f"s_cselect_b32 {t(5)}, {t(5)}, 0")
+        self.e(f"s_and_b32 {t(3)}, {self.sr('Dty')}, 1")
+        self.e(f"s_mul_i32 {t(3)}, {t(3)}, {self.sr('TilesW')}")
+        self.e(f"s_add_u32 {t(3)}, {t(3)}, {self.sr('Dtx')}")       # position inside the strip
+        self.e(f"s_and_b32 {t(4)}, {self.sr('Dty')}, -2")
+        self.e(f"s_and_b32 {t(1)}, {t(3)}, 1")
+        self.e(f"s_or_b32 {t(4)}, {t(4)}, {t(1)}")
+        self.e(f"s_lshr_b32 {t(3)}, {t(3)}, 1")
+        self.e(f"s_cmp_lg_u32 {t(5)}, 0")
+        self.e(f"s_cselect_b32 {self.sr('Dty')}, {t(4)}, {self.sr('Dty')}")
+        self.e(f"s_cselect_b32 {self.sr('Dtx')}, {t(3)}, {self.sr('Dtx')}")
 
     def patch_offsets(self):
         """Per-lane byte offsets of the 16 patch elements of the tile in D* (P cursor), relative to
@@ -1083,7 +1113,7 @@ class Kernel:
 \t.amdhsa_kernel {n}
 \t\t.amdhsa_group_segment_fixed_size 0
 \t\t.amdhsa_private_segment_fixed_size 0
-\t\t.amdhsa_kernarg_size 152
+\t\t.amdhsa_kernarg_size 168
 \t\t.amdhsa_user_sgpr_count 2
 \t\t.amdhsa_user_sgpr_kernarg_segment_ptr 1
 \t\t.amdhsa_system_sgpr_workgroup_id_x 1
@@ -1121,13 +1151,25 @@ class Kernel:
         .value_kind:     by_value
       - .offset:         148
         .size:           4
+        .value_kind:     by_value
+      - .offset:         152
+        .size:           4
+        .value_kind:     by_value
+      - .offset:         156
+        .size:           4
+        .value_kind:     by_value
+      - .offset:         160
+        .size:           4
+        .value_kind:     by_value
+      - .offset:         164
+        .size:           4
         .value_kind:     by_value"""
         return f"""  - .agpr_count:     256
     .args:
 {args}
     .group_segment_fixed_size: 0
     .kernarg_segment_align: 8
-    .kernarg_segment_size: 152
+    .kernarg_segment_size: 168
     .max_flat_workgroup_size: 256
     .name:           {self.name}
     .private_segment_fixed_size: 0

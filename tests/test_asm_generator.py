@@ -211,3 +211,145 @@ def test_h16_output_assembles_for_gfx950(tmp_path):
     subprocess.run([CLANG, "-x", "assembler", "-target", "amdgcn-amd-amdhsa", "-mcpu=gfx950",
                     "-c", str(src), "-o", str(obj)], check=True)
     assert obj.stat().st_size > 10000
+
+
+# ---------------------------------------------------------------- the tile order, executed on the CPU
+class ScalarMachine:
+    """Interpreter of the few scalar instructions the generators use for index arithmetic: runs the
+    text a generator emitted, so the tests below check the emitted code, not a restatement."""
+
+    def __init__(self):
+        self.s, self.scc = {}, 0
+
+    def val(self, x):
+        if x.startswith("s"):
+            return self.s.get(int(x[1:]), 0)
+        return int(x, 0) & 0xFFFFFFFF
+
+    def run(self, lines):
+        for line in lines:
+            line = line.strip()
+            if not line or line.startswith(";"):
+                continue
+            op, rest = line.split(None, 1)
+            a = [x.strip() for x in rest.split(",")]
+            m = 0xFFFFFFFF
+            if op == "s_mov_b32":
+                self.s[int(a[0][1:])] = self.val(a[1])
+            elif op in ("s_add_u32", "s_add_i32", "s_sub_u32", "s_sub_i32"):
+                x, y = self.val(a[1]), self.val(a[2])
+                r = x + y if "add" in op else x - y
+                self.scc = int(r > m or r < 0)
+                self.s[int(a[0][1:])] = r & m
+            elif op == "s_mul_i32":
+                self.s[int(a[0][1:])] = (self.val(a[1]) * self.val(a[2])) & m
+            elif op == "s_mul_hi_u32":
+                self.s[int(a[0][1:])] = (self.val(a[1]) * self.val(a[2])) >> 32
+            elif op in ("s_lshl_b32", "s_lshr_b32"):
+                x, n = self.val(a[1]), self.val(a[2]) & 31
+                r = (x << n) & m if op == "s_lshl_b32" else x >> n
+                self.s[int(a[0][1:])], self.scc = r, int(r != 0)
+            elif op == "s_lshr_b64":
+                lo = int(re.match(r"s\[(\d+):", a[0]).group(1))
+                src = int(re.match(r"s\[(\d+):", a[1]).group(1))
+                v = (self.s.get(src, 0) | (self.s.get(src + 1, 0) << 32)) >> (self.val(a[2]) & 63)
+                self.s[lo], self.s[lo + 1], self.scc = v & m, v >> 32, int(v != 0)
+            elif op in ("s_and_b32", "s_or_b32"):
+                x, y = self.val(a[1]), (int(a[2]) & m if re.fullmatch(r"-\d+", a[2]) else self.val(a[2]))
+                r = x & y if op == "s_and_b32" else x | y
+                self.s[int(a[0][1:])], self.scc = r, int(r != 0)
+            elif op in ("s_cmp_lt_u32", "s_cmp_gt_u32", "s_cmp_eq_u32", "s_cmp_lg_u32", "s_cmp_gt_i32"):
+                x, y = self.val(a[0]), self.val(a[1])
+                if op.endswith("i32"):
+                    x, y = (x ^ 0x80000000) - 0x80000000, (y ^ 0x80000000) - 0x80000000
+                self.scc = int({"lt": x < y, "gt": x > y, "eq": x == y, "lg": x != y}[op.split("_")[2]])
+            elif op == "s_cselect_b32":
+                self.s[int(a[0][1:])] = self.val(a[1]) if self.scc else self.val(a[2])
+            elif op == "s_bitcmp1_b32":
+                self.scc = (self.val(a[0]) >> (self.val(a[1]) & 31)) & 1
+            else:
+                raise AssertionError(f"the test's interpreter does not know {op}")
+
+
+def magic(d):
+    l = 0
+    while (1 << l) < d:
+        l += 1
+    return ((1 << (31 + l)) + d - 1) // d, 31 + l
+
+
+def decoded_tiles(k, H, W, ngroups, order_bits):
+    """(image group, tile row, tile column, live) of every column tile, as the kernel's decode()
+    computes them (one filter block, KW waves on one column tile)."""
+    th, tw = (H + 1) // 2, (W + 1) // 2
+    colgroups = th * tw * ngroups
+    k.lines = []
+    k.decode(f"s{k.S['Tp']}")
+    code = [l for l in k.lines]
+    assert not any(re.match(r"^\S+:$", l) or "s_cbranch" in l or "s_branch" in l for l in code), \
+        "decode() is dealt out over the gaps between MFMAs: it must not branch"
+    out = []
+    for t in range(colgroups // k.CW):
+        for cw in range(k.CW):
+            m = ScalarMachine()
+            S = k.S
+            m.s.update({S["H"]: H, S["W"]: W, S["TilesW"]: tw, S["Colgroups"]: colgroups, S["Cw"]: cw,
+                        S["Colblocks"]: colgroups // k.CW, S["Tp"]: t})
+            m.s[S["Mcb"]], m.s[S["Scb"]] = magic(colgroups // k.CW)
+            div = th * tw if order_bits & 1 else ngroups
+            m.s[S["Ngroups"]] = div
+            m.s[S["Mng"]], m.s[S["Sng"]] = magic(div)
+            m.s[S["Sng"]] |= 64 if order_bits & 1 else 0
+            m.s[S["Mtw"]], m.s[S["Stw"]] = magic(tw)
+            m.s[S["Stw"]] |= 64 if order_bits & 2 else 0
+            m.run(code)
+            out.append((m.s[S["Dng"]], m.s[S["Dty"]], m.s[S["Dtx"]], m.s[S["Dlive"]], m.s[S["Dkb"]]))
+    return out
+
+
+@pytest.mark.parametrize("order_bits", [0, 1, 2, 3])
+@pytest.mark.parametrize("kw,H,W,ngroups", [(4, 14, 14, 4), (2, 7, 9, 2), (4, 13, 6, 3), (2, 2, 2, 2), (4, 1, 5, 1),
+                                            (2, 56, 56, 2)])
+def test_every_tile_order_visits_every_tile_once(gen, kw, H, W, ngroups, order_bits):
+    k = gen.Kernel(kw)
+    tiles = decoded_tiles(k, H, W, ngroups, order_bits)
+    th, tw = (H + 1) // 2, (W + 1) // 2
+    assert all(live == 1 and kb == 0 for (_, _, _, live, kb) in tiles)
+    seen = {(ng, ty, tx) for (ng, ty, tx, _, _) in tiles}
+    assert len(seen) == len(tiles) == th * tw * ngroups
+    assert all(ng < ngroups and ty < th and tx < tw for (ng, ty, tx) in seen)
+    if order_bits & 1 and ngroups * th * tw > 1:
+        # neighbours on the line are neighbours in the image (or the next strip / image group begins)
+        far = sum(1 for a, b in zip(tiles, tiles[1:]) if abs(a[1] - b[1]) + abs(a[2] - b[2]) > (2 if order_bits & 2 else 1))
+        assert far <= (th + 1) * ngroups
+
+
+@pytest.mark.parametrize("tiles,ranges", [(196, 128), (196, 8), (392, 256), (49, 48), (784, 256), (3000, 1024),
+                                          (8, 8), (1000, 8), (65, 64), (12345, 256), (130, 128)])
+def test_places_of_a_line_are_a_permutation_of_each_window(gen_h16, tiles, ranges):
+    k = gen_h16.KernelH16(False)
+    k.lines = []
+    src = f"s{k.S['Tm']}"
+    k.place(src)
+    code = list(k.lines)
+    assert not any("branch" in l for l in code)
+    t5 = k.S["T"] + 5
+    mg, sh = magic(tiles)
+    placed = []
+    for on in (False, True):
+        placed = []
+        for t in range(tiles):
+            m = ScalarMachine()
+            m.s.update({k.S["Tm"]: t, k.S["PlaceM"]: mg, k.S["PlaceS"]: sh | (64 if on else 0),
+                        k.S["PlaceG"]: ranges, k.S["PlaceTn"]: tiles})
+            m.run(code)
+            placed.append(m.s[t5])
+        if not on:
+            assert placed == list(range(tiles))
+    assert sorted(placed) == list(range(tiles))
+    for x in range(8):  # inside its XCD's window, the tiles in which a range begins first
+        lo, nxt = (x * tiles + 7) // 8, ((x + 1) * tiles + 7) // 8
+        window = placed[lo:nxt]
+        assert sorted(window) == list(range(lo, nxt))
+        begins = [t for t in range(lo, nxt) if (t + 1) * ranges // tiles > t * ranges // tiles]
+        assert [placed[t] for t in begins] == list(range(lo, lo + len(begins)))

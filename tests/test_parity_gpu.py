@@ -763,6 +763,39 @@ def test_reduced_precision_on_shapes_outside_the_tiling(ocn, oracle, torch_gpu, 
     assert rel64 <= REL_L2_DIRECT_REDUCED[prec], f"rel-L2 vs fp64 direct {rel64:.3e}"
 
 
+@pytest.mark.parametrize("prec", ["f32", "f16"])
+@pytest.mark.parametrize("N,C,H,W,K", [(128, 64, 14, 14, 256), (64, 16, 41, 41, 128), (96, 32, 13, 22, 64),
+                                       (64, 32, 27, 9, 320), (32, 512, 7, 7, 512)])
+def test_every_tile_order_computes_the_same_layer(ocn, oracle, torch_gpu, prec, N, C, H, W, K):
+    # The order in which the assembly kernels walk through the image (opencnn_set_tile_order: image
+    # group or spatial tile fastest, rows or zigzag strips, places by starting time) only changes
+    # which tiles are cut between workgroups: every output element is written, inside the tensor,
+    # and equals the default order's up to the association of the channel sum.
+    print(f"tile orders {prec} N={N} C={C} H={H} W={W} K={K}", flush=True)
+    x, w = make_tensors(ocn, N, C, H, W, K)
+    r = Runner(ocn, torch_gpu, x, w)
+    results = {}
+    try:
+        ocn.set_operand_precision({"f32": ocn.F32, "f16": ocn.F16}[prec])
+        for order in (7, 0, 1, 2, 3, 5):
+            ocn.set_tile_order(order)
+            r.raw.fill_(float("nan"))
+            results[order] = r.split()
+            assert "_asm_" in ocn.last_kernel()
+    finally:
+        ocn.set_tile_order(7)
+        ocn.set_operand_precision(ocn.F32)
+    want = oracle.direct_conv_f64(x, w)
+    for order, y in results.items():
+        assert not np.isnan(y).any(), f"order {order}: an output element was never written"
+        rel64, _, _ = oracle.compare(y, want)
+        assert rel64 <= {"f32": 1e-5, "f16": 2e-3}[prec], f"order {order}: rel-L2 vs fp64 direct {rel64:.3e}"
+        rel, _, _ = oracle.compare(y, results[7])
+        assert rel <= 3e-6, f"order {order}: rel-L2 vs the default order {rel:.3e}"
+    with pytest.raises(ocn.OpenCNNError):
+        ocn.set_tile_order(8)
+
+
 def test_non_default_stream(ocn, oracle, torch_gpu):
     print("stream", flush=True)
     torch = torch_gpu
