@@ -341,3 +341,30 @@ def test_a_wait_that_gives_up_is_reported(ocn, oracle, torch_gpu):
         ocn.conv_forward_pretransformed(r.xd, r.ws, r.yd, N, C, H, W, K)
         assert np.array_equal(r.result(), want)
     ocn.check_status()
+
+
+def test_timing_entry_point(ocn, oracle, torch_gpu):
+    # opencnn_time_forward, the library-side twin of the reference's timing loop
+    # (src/openCNN_winograd.cu:426-444): plausible times, only the loops asked for run, and the
+    # tensors it leaves behind are the layer's.
+    print("time_forward", flush=True)
+    N, C, H, W, K = 32, 16, 12, 12, 64
+    x, w = make_tensors(ocn, N, C, H, W, K)
+    r = Runner(ocn, torch_gpu, x, w)
+    total, main, fx = ocn.time_forward(r.xd, r.wd, r.yd, r.ws, N, C, H, W, K, warmup=2, iters=20)
+    assert 0 < fx < total and 0 < main < total and total < 1.0
+    assert total <= 1.5 * (main + fx)
+    check_against_oracle(oracle, r.result(), x, w)
+    only_main = ocn.time_forward(r.xd, r.wd, r.yd, r.ws, N, C, H, W, K, warmup=0, iters=5, parts=("main",))
+    assert only_main[0] == 0 and only_main[1] > 0 and only_main[2] == 0
+    for bad in (dict(iters=0), dict(warmup=-1)):
+        with pytest.raises(ocn.OpenCNNError):
+            ocn.time_forward(r.xd, r.wd, r.yd, r.ws, N, C, H, W, K, **bad)
+    try:  # the process-wide precision applies, as for convolutionForward
+        ocn.set_operand_precision(ocn.BF16)
+        ocn.time_forward(r.xd, r.wd, r.yd, r.ws, N, C, H, W, K, warmup=1, iters=3)
+        assert "bf16" in ocn.last_kernel()
+    finally:
+        ocn.set_operand_precision(ocn.F32)
+    torch_gpu.cuda.synchronize()
+    ocn.check_status()
