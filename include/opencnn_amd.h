@@ -331,8 +331,8 @@ int opencnn_time_forward(const float *in, const float *w, float *out, float *Ww,
  * the L2 of its XCD because a neighbouring tile has just read it.  Results do not depend on it.
  * Bits: 1 = neighbouring column tiles are neighbouring spatial tiles (else: the same spatial tile
  * of the next 32 batch elements), 2 = spatial tiles numbered in zigzag strips of two tile rows
- * (else row by row), 4 = fp16 / bf16 kernels: the tiles that an XCD's workgroups start with lie
- * together in the image, the tiles they go on with beside them.  Default 7; 0 is the order of
+ * (else row by row), 4 = the tiles that an XCD's workgroups start with lie together in the image,
+ * the tiles they go on with beside them.  Default 7; 0 is the order of
  * the first version of the kernels, kept for measurements (profiles/).
  */
 int opencnn_set_tile_order(int bits);

@@ -267,7 +267,7 @@ struct AsmKernArgs {
   long long* timeline;     // 64 entries per workgroup, or null
   unsigned* status;        // status word of the flag set (a wave that gives up a wait stores 1)
   uint32_t wait_polls;     // polls after which a wait for a flag gives up
-  // fp16 / bf16 kernels: the places of a line's tiles (KernelH16.place): magic number of the
+  // the places of a line's tiles (Kernel.place in gen_wino_f32_asm.py): magic number of the
   // tiles on the line (bit 6 of the shift switches the places on), ranges and tiles on the line
   uint32_t m_place, s_place;
   int32_t place_ranges, place_tiles;
@@ -511,8 +511,8 @@ struct AsmLaunch {
   // Spatial tiles numbered in strips of two tile rows, zigzag, instead of row by row (fp32
   // N=64 C=K=64 56x56: 137.4 -> 129.3 MB, -0.5 % time).
   bool strips = g_tile_order.load() & 2;
-  // fp16 / bf16 kernels: the tiles in work from the start get the first places of an XCD's window
-  // (KernelH16.place; 93.3 -> 82.4 MB on the fp16 benchmark layer).
+  // The tiles in work from the start get the first places of an XCD's window (Kernel.place;
+  // 93.3 -> 82.4 MB on the fp16 benchmark layer).
   bool tile_places = g_tile_order.load() & 4;
 };
 
@@ -549,13 +549,16 @@ int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmLaunch& l, hipStream_
     ka.k_real = (int32_t)vt;
     chunk_divisor = (uint32_t)vt;
   }
-  if (l.filters >= 0) {
+  {
     // the line of tiles the ranges are cut from, before its weights: one per filter block, or one
     const long long line_tiles = l.lockstep_log2 >= 0 ? a.nblocks >> l.lockstep_log2 : a.nblocks;
     ka.place_tiles = (int32_t)line_tiles;
     ka.place_ranges = ranges;
     magic_divisor((uint32_t)line_tiles, &ka.m_place, &ka.s_place);
-    if (l.tile_places && !l.packed && !l.natural_order && ranges % 8 == 0 && ranges <= line_tiles &&
+    // (a tile switch of the fp32 kernels carries the five divisions of place() between its MFMAs:
+    // not worth it where a tile is only a few units long)
+    if (l.tile_places && !l.packed && !l.natural_order && (l.filters >= 0 || chunks >= 4) && ranges % 8 == 0 &&
+        ranges <= line_tiles &&
         line_tiles * ranges + ranges <= kMaxElems && line_tiles * 8 <= kMaxElems)
       ka.s_place |= 64;
   }

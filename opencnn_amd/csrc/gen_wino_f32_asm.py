@@ -52,7 +52,7 @@ A wait for a flag is bounded so that a bug or a workgroup that never becomes res
 hang the GPU.  A wave that gives up writes 1 to the status word and goes on with whatever the
 output tensor holds: the launch's result is wrong, every wave still ends, and the host finds
 the word at its next call (api.hip: the call fails and the flags are cleared).  The last four
-ints (the places of the tiles of a line in the image) are read by the fp16 / bf16 kernels only.
+ints describe the places of the tiles of a line in the image (place()).
 
 Usage: gen_wino_f32_asm.py > wino_f32_asm.s
 """
@@ -93,6 +93,7 @@ def a(i, n=1):
 
 class Kernel:
     K_REAL = "Kreal"  # the scalar register with the real filter count (ragged K)
+    CW_IS_FREE = False  # lane_setup and decode read Cw (the wave's column tile inside the workgroup tile)
 
     def __init__(self, KW, ragged=False, packed=False):
         """ragged: shapes outside N % 32 == 0, K % 32 == 0, C % 8 == 0.  Groups and chunks are
@@ -153,6 +154,11 @@ class Kernel:
         self.S["Yt"] = S.get("Yt", 2, 2)
         self.S["Fl"] = S.get("Fl", 2, 2)
         self.S["T"] = S.get("T", 8, 2)  # temporaries T0..T7 (T6:T7 = division pair)
+        # place(): the magic number of the line's tile count in two user registers that are free, the
+        # ranges on the line in GridPerXcd (dead after head) and the tile count in a register of
+        # its own, or in Cw where nothing reads that after head (CW_IS_FREE)
+        self.S.update(PlaceM=3, PlaceS=7, PlaceG=self.S["GridPerXcd"])
+        self.S["PlaceTn"] = self.S["Cw"] if self.CW_IS_FREE else S.get("PlaceTn")
         self.sgpr_count = S.next
 
     def alloc_vgprs(self):
@@ -190,16 +196,64 @@ class Kernel:
         self.e(f"s_lshr_b64 {s(t6, 2)}, {s(t6, 2)}, {sh}")
         self.e(f"s_mov_b32 {dst}, {s(t6)}")
 
+    # ------------------------------------------------------------------ where a tile of the line lies
+    # The workgroups of an XCD walk through a window of neighbouring tiles of the line.  About
+    # G / Tn of them (G ranges on a line of Tn tiles) are in work from the start - the tiles in
+    # which a range begins - and the others are taken up one tile time later.  The patch lines a
+    # tile shares with its neighbours in the image are only found in L2 while those neighbours
+    # are in work too: an XCD's 4 MB do not keep a tile's patches (next to the transformed
+    # filter) until a later tile asks for them.  So the tiles that are in work from the start get
+    # the first places of their window and the later ones the rest: two compact blocks of the
+    # image instead of an interleaved pattern.  place(t), with E(t) = t * G / Tn (the ranges that
+    # begin in front of tile t, for equal ranges) and the window of XCD x = tiles
+    # [ceil(x * Tn / 8), ceil((x + 1) * Tn / 8)):
+    #   begins a range (E(t + 1) > E(t)):  lo + E(t) - E(lo)
+    #   else:                              t + (E(next lo) - E(lo)) - (E(t) - E(lo))
+    # a permutation of every window whatever the real range boundaries are (they only decide how
+    # well it works).  Bit 6 of the magic shift switches it on (64-bit shifts ignore the bit).
+    def place(self, T):
+        """t5 = the place of tile T of the line (T itself when the host has not asked for places)."""
+        t, e = self.t, self.e
+        pm, ps, g, tn = self.sr("PlaceM"), self.sr("PlaceS"), self.sr("PlaceG"), self.sr("PlaceTn")
+        e(f"s_lshl_b32 {t(0)}, {T}, 3")
+        self.div(t(1), t(0), pm, ps)                      # x: the window
+        e(f"s_mul_i32 {t(2)}, {t(1)}, {tn}")
+        e(f"s_add_u32 {t(3)}, {t(2)}, {tn}")
+        e(f"s_add_u32 {t(2)}, {t(2)}, 7")
+        e(f"s_lshr_b32 {t(2)}, {t(2)}, 3")                # lo
+        e(f"s_add_u32 {t(3)}, {t(3)}, 7")
+        e(f"s_lshr_b32 {t(3)}, {t(3)}, 3")                # lo of the next window
+        e(f"s_mul_i32 {t(0)}, {t(2)}, {g}")
+        self.div(t(4), t(0), pm, ps)                      # E(lo)
+        e(f"s_mul_i32 {t(0)}, {t(3)}, {g}")
+        self.div(t(3), t(0), pm, ps)                      # E(next lo)
+        e(f"s_sub_u32 {t(3)}, {t(3)}, {t(4)}")            # ranges that begin in the window
+        e(f"s_mul_i32 {t(0)}, {T}, {g}")
+        self.div(t(1), t(0), pm, ps)                      # E(t)
+        e(f"s_add_u32 {t(0)}, {t(0)}, {g}")
+        self.div(t(5), t(0), pm, ps)                      # E(t + 1)
+        e(f"s_sub_u32 {t(4)}, {t(1)}, {t(4)}")            # E(t) - E(lo)
+        e(f"s_add_u32 {t(2)}, {t(2)}, {t(4)}")            # the place of a tile in which a range begins
+        e(f"s_add_u32 {t(3)}, {T}, {t(3)}")
+        e(f"s_sub_u32 {t(3)}, {t(3)}, {t(4)}")            # the place of a later tile
+        e(f"s_cmp_gt_u32 {t(5)}, {t(1)}")
+        e(f"s_cselect_b32 {t(5)}, {t(2)}, {t(3)}")
+        e(f"s_bitcmp1_b32 {ps}, 6")
+        e(f"s_cselect_b32 {t(5)}, {t(5)}, {T}")
+
     def split_tile(self, T):
-        """Workgroup tile T -> Dkb (filter block) and T0 (column block): filter-block major."""
+        """Workgroup tile T of the line -> Dkb (filter block) and T0 (column block) of its place:
+        filter-block major."""
         t = self.t
-        self.div(self.sr("Dkb"), T, self.sr("Mcb"), self.sr("Scb"))
+        self.place(T)
+        self.div(self.sr("Dkb"), t(5), self.sr("Mcb"), self.sr("Scb"))
         self.e(f"s_mul_i32 {t(0)}, {self.sr('Dkb')}, {self.sr('Colblocks')}")
-        self.e(f"s_sub_u32 {t(0)}, {T}, {t(0)}")  # column block
+        self.e(f"s_sub_u32 {t(0)}, {t(5)}, {t(0)}")  # column block
 
     def filter_block(self, dst, T):
-        """dst = filter block of workgroup tile T (may use T0, T1)."""
-        self.div(dst, T, self.sr("Mcb"), self.sr("Scb"))
+        """dst = filter block of workgroup tile T (may use T0 .. T5)."""
+        self.place(T)
+        self.div(dst, self.t(5), self.sr("Mcb"), self.sr("Scb"))
 
     def decode(self, T):
         """Workgroup tile T -> Dkb (filter block), Dlive, Dng, Dty, Dtx of this wave's column tile."""
@@ -955,6 +1009,12 @@ class Kernel:
         e(f"s_cmp_eq_u32 {self.sr('GridPerXcd')}, 0")
         e(f"s_cselect_b32 {self.sr('L')}, s2, {t(0)}")
         self.unit_range(self.range_owner())
+        # the arguments of place(), into registers that are free from here on
+        e(f"s_load_dword {self.sr('PlaceM')}, s[0:1], 0x94")
+        e(f"s_load_dword {self.sr('PlaceS')}, s[0:1], 0x98")
+        e(f"s_load_dword {self.sr('PlaceG')}, s[0:1], 0x9c")
+        e(f"s_load_dword {self.sr('PlaceTn')}, s[0:1], 0xa0")
+        e("s_waitcnt lgkmcnt(0)")
         for n in ("Tp", "Tq"):
             e(f"s_mov_b32 {self.sr(n)}, {self.sr('Tm')}")
         for n in ("Cp", "Cq"):

@@ -54,6 +54,7 @@ class Wait:
 class KernelH16(Kernel):
     SLAB_CHANNELS = 4
     K_REAL = "Q"  # the argument slot Q (twice the chunks per tile in the fp32 kernels) carries K here
+    CW_IS_FREE = True  # one column tile per workgroup: Cw is zero and nothing here reads it
 
     def __init__(self, bf16, ragged=False, packed=False):
         """ragged: shapes outside N % 32 == 0, C % 16 == 0, K % 32 == 0 (masked lanes and rows, a
@@ -101,10 +102,6 @@ class KernelH16(Kernel):
         self.S["Lr"] = S.get("Lr")
         self.S["Kbf"] = S.get("Kbf")
         self.sgpr_count = S.next
-        # place(): the magic number of the line's tile count in two user registers that are free;
-        # the tile count and the ranges on the line in Cw (a workgroup has one column tile here)
-        # and GridPerXcd, both dead after Kernel.head
-        self.S.update(PlaceM=3, PlaceS=7, PlaceG=self.S["GridPerXcd"], PlaceTn=self.S["Cw"])
 
     def head(self):
         """After the common set-up: the time-aligned chunk order.  A workgroup's g-th unit works on
@@ -120,11 +117,6 @@ class KernelH16(Kernel):
         They live in argument registers that are dead after this set-up."""
         super().head()
         t, e = self.t, self.e
-        e(f"s_load_dword {self.sr('PlaceM')}, s[0:1], 0x94")
-        e(f"s_load_dword {self.sr('PlaceS')}, s[0:1], 0x98")
-        e(f"s_load_dword {self.sr('PlaceG')}, s[0:1], 0x9c")
-        e(f"s_load_dword {self.sr('PlaceTn')}, s[0:1], 0xa0")
-        e("s_waitcnt lgkmcnt(0)")
         self.S.update(N1=self.S["Kreal"], Sfull=self.S["UnitsQ"], Tlast=self.S["UnitsRem"], Nlast=self.S["Mch"])
         e(f"s_sub_u32 {t(0)}, {self.sr('Chunks')}, {self.sr('Cm')}")
         e(f"s_cmp_eq_u32 {self.sr('Cm')}, 0")
@@ -287,51 +279,6 @@ class KernelH16(Kernel):
         self.e(f"s_sub_u32 {t(0)}, {self.sr('Colblocks')}, 1")
         self.e(f"s_and_b32 {self.sr('Kbf')}, {self.sr('L')}, {t(0)}")
         return self.sr("Lr")
-
-    # ------------------------------------------------------------------ where a tile of the line lies
-    # The workgroups of an XCD walk through a window of neighbouring tiles of the line.  About
-    # G / Tn of them (G ranges on a line of Tn tiles) are in work from the start - the tiles in
-    # which a range begins - and the others are taken up one tile time later.  The patch lines a
-    # tile shares with its neighbours in the image are only found in L2 while those neighbours
-    # are in work too: an XCD's 4 MB do not keep a tile's patches (next to the transformed
-    # filter) until a later tile asks for them.  So the tiles that are in work from the start get
-    # the first places of their window and the later ones the rest: two compact blocks of the
-    # image instead of an interleaved pattern.  place(t), with E(t) = t * G / Tn (the ranges that
-    # begin in front of tile t, for equal ranges) and the window of XCD x = tiles
-    # [ceil(x * Tn / 8), ceil((x + 1) * Tn / 8)):
-    #   begins a range (E(t + 1) > E(t)):  lo + E(t) - E(lo)
-    #   else:                              t + (E(next lo) - E(lo)) - (E(t) - E(lo))
-    # a permutation of every window whatever the real range boundaries are (they only decide how
-    # well it works).  Bit 6 of the magic shift switches it on (64-bit shifts ignore the bit).
-    def place(self, T):
-        """t5 = the place of tile T of the line (T itself when the host has not asked for places)."""
-        t, e = self.t, self.e
-        pm, ps, g, tn = self.sr("PlaceM"), self.sr("PlaceS"), self.sr("PlaceG"), self.sr("PlaceTn")
-        e(f"s_lshl_b32 {t(0)}, {T}, 3")
-        self.div(t(1), t(0), pm, ps)                      # x: the window
-        e(f"s_mul_i32 {t(2)}, {t(1)}, {tn}")
-        e(f"s_add_u32 {t(3)}, {t(2)}, {tn}")
-        e(f"s_add_u32 {t(2)}, {t(2)}, 7")
-        e(f"s_lshr_b32 {t(2)}, {t(2)}, 3")                # lo
-        e(f"s_add_u32 {t(3)}, {t(3)}, 7")
-        e(f"s_lshr_b32 {t(3)}, {t(3)}, 3")                # lo of the next window
-        e(f"s_mul_i32 {t(0)}, {t(2)}, {g}")
-        self.div(t(4), t(0), pm, ps)                      # E(lo)
-        e(f"s_mul_i32 {t(0)}, {t(3)}, {g}")
-        self.div(t(3), t(0), pm, ps)                      # E(next lo)
-        e(f"s_sub_u32 {t(3)}, {t(3)}, {t(4)}")            # ranges that begin in the window
-        e(f"s_mul_i32 {t(0)}, {T}, {g}")
-        self.div(t(1), t(0), pm, ps)                      # E(t)
-        e(f"s_add_u32 {t(0)}, {t(0)}, {g}")
-        self.div(t(5), t(0), pm, ps)                      # E(t + 1)
-        e(f"s_sub_u32 {t(4)}, {t(1)}, {t(4)}")            # E(t) - E(lo)
-        e(f"s_add_u32 {t(2)}, {t(2)}, {t(4)}")            # the place of a tile in which a range begins
-        e(f"s_add_u32 {t(3)}, {T}, {t(3)}")
-        e(f"s_sub_u32 {t(3)}, {t(3)}, {t(4)}")            # the place of a later tile
-        e(f"s_cmp_gt_u32 {t(5)}, {t(1)}")
-        e(f"s_cselect_b32 {t(5)}, {t(2)}, {t(3)}")
-        e(f"s_bitcmp1_b32 {ps}, 6")
-        e(f"s_cselect_b32 {t(5)}, {t(5)}, {T}")
 
     def split_tile(self, T):
         """T -> T0 (column block), Dkb (filter block)."""

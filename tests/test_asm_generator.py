@@ -30,7 +30,7 @@ VARIANTS = [(False, False), (True, False), (True, True)]  # (ragged, packed)
 def test_register_budget(gen, kw, ragged, packed):
     k = gen.Kernel(kw, ragged, packed)
     assert k.vgpr_count <= 256          # arch VGPRs; the 256 accumulators are AGPRs
-    assert k.sgpr_count <= 96           # + VCC and the reserved registers of the target = 102
+    assert k.sgpr_count <= 100          # s0 .. s101 less VCC, which the kernel descriptor reserves (the assembler checks too)
     assert len(set(k.MP)) == 64         # landing registers of a published partial tile
     live_at_boundary = set()
     for name in ("U0", "U1", "D0", "D1", "VA", "VOFF", "Off", "Eff"):
@@ -149,7 +149,7 @@ def gen_h16(gen):
 def test_h16_register_budget(gen_h16, bf16, ragged, packed):
     k = gen_h16.KernelH16(bf16, ragged, packed)
     assert k.vgpr_count <= 256
-    assert k.sgpr_count <= 98
+    assert k.sgpr_count <= 100
     assert len(set(k.MP)) == 64
     live_at_boundary = set()
     for name, n in (("U", 64), ("DA0", 16), ("DB0", 16), ("DA1", 16), ("DB1", 16), ("VOFF", 16),
@@ -326,8 +326,9 @@ def test_every_tile_order_visits_every_tile_once(gen, kw, H, W, ngroups, order_b
 
 @pytest.mark.parametrize("tiles,ranges", [(196, 128), (196, 8), (392, 256), (49, 48), (784, 256), (3000, 1024),
                                           (8, 8), (1000, 8), (65, 64), (12345, 256), (130, 128)])
-def test_places_of_a_line_are_a_permutation_of_each_window(gen_h16, tiles, ranges):
-    k = gen_h16.KernelH16(False)
+@pytest.mark.parametrize("family", ["f32_kw2", "f32_kw4", "f16"])
+def test_places_of_a_line_are_a_permutation_of_each_window(gen, gen_h16, family, tiles, ranges):
+    k = {"f32_kw2": lambda: gen.Kernel(2), "f32_kw4": lambda: gen.Kernel(4), "f16": lambda: gen_h16.KernelH16(False)}[family]()
     k.lines = []
     src = f"s{k.S['Tm']}"
     k.place(src)
