@@ -9,9 +9,10 @@
  * them per call instead), the code objects of its assembly kernels (embedded in the library,
  * loaded once per device by opencnn_init or the first launch), 1.5 MB of static device memory
  * that the balanced split uses to hand tiles over between workgroups (48 sets of flags, zero
- * between launches; see opencnn_set_balanced_split), 200 bytes of pinned host memory per device
- * that the kernels report a failed hand-over in (opencnn_check_status), and a host-side record of
- * the transformed filters it wrote (opencnn_filter_transform).
+ * between launches; see opencnn_set_balanced_split), per device 200 bytes of pinned host memory
+ * that the kernels report a failed hand-over in (opencnn_check_status) and 32 events, all made by
+ * opencnn_init or the first launch on the device, and a host-side record of the transformed
+ * filters it wrote (opencnn_filter_transform).
  * All entry points return a hipError_t value as int (0 == hipSuccess); launches are
  * asynchronous on the selected stream, exactly like the reference, which returns
  * cudaGetLastError() right after its two launches

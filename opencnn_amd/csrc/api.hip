@@ -151,6 +151,10 @@ int device_state(DeviceState** out) {
     if ((e = hipHostGetDevicePointer(&dev_view, host, 0)) != hipSuccess) return (int)e;
     k.status_host = static_cast<volatile unsigned*>(host);
     k.status_dev = static_cast<unsigned*>(dev_view);
+    // the events that tell when a stream's flag set is idle: created here, so that no launch
+    // (opencnn_conv_forward_static in particular) ever creates anything
+    for (int i = 0; i < opencnn::kEagerSets; ++i)
+      if ((e = hipEventCreateWithFlags(&k.owners[i].idle, hipEventDisableTiming)) != hipSuccess) return (int)e;
     // 64 KB of dynamic LDS for KW = 2 is the default limit exactly; nothing to raise
     k.ready = true;
     g_device_ready[dev].store(true);
@@ -231,8 +235,7 @@ void flag_set_launched(DeviceState* ds, int set, hipStream_t st) {
   std::lock_guard<std::mutex> lock(ds->flag_mu);
   FlagSetOwner& o = ds->owners[set];
   if (ds->pressure && set < opencnn::kEagerSets) {
-    if (o.idle == nullptr && hipEventCreateWithFlags(&o.idle, hipEventDisableTiming) != hipSuccess) o.idle = nullptr;
-    o.idle_recorded = o.idle != nullptr && hipEventRecord(o.idle, st) == hipSuccess;
+    o.idle_recorded = hipEventRecord(o.idle, st) == hipSuccess;
   }
   --o.calls_in_flight;
 }
