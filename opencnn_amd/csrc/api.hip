@@ -560,7 +560,7 @@ int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmLaunch& l, hipStream_
     magic_divisor((uint32_t)line_tiles, &ka.m_place, &ka.s_place);
     // (a tile switch of the fp32 kernels carries the five divisions of place() between its MFMAs:
     // not worth it where a tile is only a few units long)
-    if (l.tile_places && !l.packed && !l.natural_order && (l.filters >= 0 || chunks >= 4) && ranges % 8 == 0 &&
+    if (l.tile_places && !l.natural_order && (l.filters >= 0 || chunks >= 4) && ranges % 8 == 0 &&
         ranges <= line_tiles &&
         line_tiles * ranges + ranges <= kMaxElems && line_tiles * 8 <= kMaxElems)
       ka.s_place |= 64;
