@@ -234,8 +234,9 @@ void flag_set_launched(DeviceState* ds, int set, hipStream_t st) {
   if (set < 0 || set >= opencnn::kSyncSets) return;
   std::lock_guard<std::mutex> lock(ds->flag_mu);
   FlagSetOwner& o = ds->owners[set];
-  if (ds->pressure && set < opencnn::kEagerSets) {
-    o.idle_recorded = hipEventRecord(o.idle, st) == hipSuccess;
+  if (set < opencnn::kEagerSets) {
+    // without pressure nothing is recorded, and an earlier record no longer covers the set's last launch
+    o.idle_recorded = ds->pressure && hipEventRecord(o.idle, st) == hipSuccess;
   }
   --o.calls_in_flight;
 }
@@ -250,6 +251,7 @@ int release_flag_set(DeviceState* ds, hipStream_t st) {
     if (o.used && o.stream == st && o.calls_in_flight == 0) {
       o.used = false;
       o.idle_recorded = false;
+      ds->pressure = false;  // a set is free again: no events until the sets run out once more
     }
   }
   return 0;
