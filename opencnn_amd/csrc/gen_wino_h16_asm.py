@@ -41,7 +41,7 @@ import sys
 from gen_wino_f32_asm import MERGE_POSITIONS, Alloc, Kernel, a, s, v
 
 RING = 8   # B operands in registers (positions)
-LEAD = 6   # positions the LDS reads run ahead of the MFMAs
+LEAD = 3   # positions the LDS reads run ahead of the MFMAs
 
 
 class Wait:
