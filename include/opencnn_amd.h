@@ -42,7 +42,7 @@ extern "C" {
 /* Layout of the transformed-filter buffer written by opencnn_filter_transform. */
 enum {
   OPENCNN_WW_REFERENCE = 0, /* [filt_c][16][filt_k], position p = i*4+j (src/FX_m2.cu:84) */
-  OPENCNN_WW_MFMA = 1       /* [kp/32][cp/4][16][2][32][2], kp / cp = filt_k / filt_c rounded up to 32 / 8,
+  OPENCNN_WW_MFMA = 1       /* [kp/32][cp/4][8][2][32][2][2], kp / cp = filt_k / filt_c rounded up to 32 / 8,
                                padding zero: what the fused kernels read */
 };
 

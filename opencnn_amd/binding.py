@@ -382,12 +382,12 @@ def synth_filter(k, c, seed, layout=FILTER_CRSK, dist=DIST_NORMAL, p0=0.0, p1=No
 
 
 def unswizzle_ww(ww_mfma: np.ndarray, filt_c: int, filt_k: int) -> np.ndarray:
-    """Reorder a host copy of an OPENCNN_WW_MFMA buffer ([kp/32][cp/4][16][2][32][2], kp / cp =
+    """Reorder a host copy of an OPENCNN_WW_MFMA buffer ([kp/32][cp/4][8][2][32][2][2], kp / cp =
     filt_k / filt_c rounded up to 32 / 8) into the reference's [c][16][k] order
     (src/FX_m2.cu:84).  Pure permutation, no arithmetic; the zero padding is dropped."""
     kp, cp = -(-filt_k // 32) * 32, -(-filt_c // 8) * 8
     a = np.asarray(ww_mfma, dtype=np.float32).reshape(-1)[:kp * cp * 16]  # a workspace may be larger
-    a = a.reshape(kp // 32, cp // 4, 16, 2, 32, 2)
-    # axes: kg, q, p, h, k32, s ; c = 4q + 2s + h ; k = 32kg + k32
-    a = a.transpose(1, 5, 3, 2, 0, 4)  # q, s, h, p, kg, k32
+    a = a.reshape(kp // 32, cp // 4, 8, 2, 32, 2, 2)
+    # axes: kg, q, p/2, h, k32, p%2, s ; c = 4q + 2s + h ; k = 32kg + k32
+    a = a.transpose(1, 6, 3, 2, 5, 0, 4)  # q, s, h, p/2, p%2, kg, k32
     return np.ascontiguousarray(a.reshape(cp, 16, kp)[:filt_c, :, :filt_k])

@@ -33,6 +33,7 @@ namespace opencnn {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v2f __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 typedef unsigned int v2u __attribute__((ext_vector_type(2)));
 
 struct ConvArgs {
@@ -182,8 +183,11 @@ __device__ __forceinline__ void load_u(const ConvArgs& a, const WaveTile& w, int
   const int qd = quad < Q ? quad : Q - 1;
   const int soff = (w.kg * Q + qd) * (16 * 64 * 8);
 #pragma unroll
-  for (int p = 0; p < 16; ++p)
-    u[p] = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(ru, lane * 8 + p * 512, soff, 0));
+  for (int p = 0; p < 16; p += 2) {
+    const v4f pair = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(ru, lane * 16 + p * 512, soff, 0));
+    u[p] = v2f{pair[0], pair[1]};
+    u[p + 1] = v2f{pair[2], pair[3]};
+  }
 }
 
 // Output transform and store.  Accumulator register r of lane (hsel, nl) is row
@@ -605,8 +609,11 @@ __device__ __forceinline__ void load_u_s(const ConvArgs& a, int kg, int lane, v2
   const __amdgpu_buffer_rsrc_t ru = make_rsrc(a.usw, (unsigned)((size_t)a.C * 16 * a.K * sizeof(float)));
   const int soff = __builtin_amdgcn_readfirstlane((kg * Q + quad) * (16 * 64 * 8));
 #pragma unroll
-  for (int p = 0; p < 16; ++p)
-    u[p] = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(ru, lane * 8 + p * 512, soff, 0));
+  for (int p = 0; p < 16; p += 2) {
+    const v4f pair = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(ru, lane * 16 + p * 512, soff, 0));
+    u[p] = v2f{pair[0], pair[1]};
+    u[p + 1] = v2f{pair[2], pair[3]};
+  }
 }
 
 template <int KW, bool BALANCED, bool SCALAR_PATCH>

@@ -62,10 +62,11 @@ __global__ void __launch_bounds__(256) fx_reference_layout(const float* __restri
 }
 
 // MFMA-operand layout read by the fused kernel:
-//   Usw[kg][q][p][h][k32][s],  k = kg*32 + k32,  c = 4*q + 2*s + h
-// so that lane (h*32 + k32) of a wave fetches, with one 8-byte load per position p, the A
-// operand of two consecutive v_mfma_f32_32x32x2_f32 steps (channels 4q+h and 4q+2+h).
-// Thread = (k, q, h): transforms the two channels c = 4q+h and 4q+2+h and writes float2.
+//   Usw[kg][q][p/2][h][k32][p%2][s],  k = kg*32 + k32,  c = 4*q + 2*s + h
+// so that lane (h*32 + k32) of a wave fetches, with one 16-byte load per pair of positions
+// (p, p+1), the A operands of two consecutive v_mfma_f32_32x32x2_f32 steps (channels 4q+h and
+// 4q+2+h) of both positions.
+// Thread = (k, q, h): transforms the two channels c = 4q+h and 4q+2+h and writes float4.
 // grid (ceil(K/128), Cpad/4), block 256 = 2 h x 128 k.
 //
 // Shapes the reference does not take (K not a multiple of 32, C not a multiple of 8) are
@@ -94,10 +95,10 @@ __global__ void __launch_bounds__(256) fx_mfma_layout(const float* __restrict__ 
     }
   }
   const int kg = k >> 5, k32 = k & 31;
-  float2* o = reinterpret_cast<float2*>(Usw) +
-              (((size_t)kg * gridDim.y + q) * 16) * 64 + h * 32 + k32;
+  float4* o = reinterpret_cast<float4*>(Usw) +
+              (((size_t)kg * gridDim.y + q) * 8) * 64 + h * 32 + k32;
 #pragma unroll
-  for (int p = 0; p < 16; ++p) o[(size_t)p * 64] = make_float2(U0[p], U1[p]);
+  for (int p = 0; p < 16; p += 2) o[(size_t)(p >> 1) * 64] = make_float4(U0[p], U1[p], U0[p + 1], U1[p + 1]);
 }
 
 // Reduced-precision MFMA-operand layout read by the fp16 / bf16 fused kernel:

@@ -164,7 +164,7 @@ class Kernel:
     def alloc_vgprs(self):
         V = Alloc(1, 256)
         self.V = {}
-        for n, cnt, al in [("Lane", 1, 1), ("LaneX", 1, 1), ("Lane8", 1, 1), ("Lane8b", 1, 1),
+        for n, cnt, al in [("Lane", 1, 1), ("LaneX", 1, 1), ("LaneU", 1, 1), ("LaneUb", 1, 1),
                            ("Lds", 1, 1), ("LdsWr", 1, 1), ("Zero", 1, 1), ("One", 1, 1), ("Oob", 1, 1),
                            ("Tmp", 4, 1),
                            ("Off", 4, 1), ("Eff", 4, 1), ("VOFF", 16, 1),
@@ -531,8 +531,12 @@ class Kernel:
 
     # ------------------------------------------------------------------ vector pieces
     def load_u(self, dst, p, soff):
-        lane = self.vr("Lane8") if p < 8 else self.vr("Lane8b")
-        self.e(f"buffer_load_dwordx2 {self.vr(dst, 2 * p, 2)}, {lane}, {self.sr('RsrcU', 4)}, {soff} offen offset:{(p % 8) * 512}")
+        """A operands of positions p and p + 1 (two MFMA steps each): one 16-byte load, issued in
+        the slot of the even position."""
+        if p % 2:
+            return
+        lane = self.vr("LaneU") if p < 8 else self.vr("LaneUb")
+        self.e(f"buffer_load_dwordx4 {self.vr(dst, 2 * p, 4)}, {lane}, {self.sr('RsrcU', 4)}, {soff} offen offset:{(p % 8) * 512}")
 
     def load_patch(self, dst, p):
         self.e(f"buffer_load_dword {self.vr(dst, p)}, {self.vr('VOFF', p)}, {self.sr('RsrcX', 4)}, 0 offen")
@@ -686,7 +690,7 @@ class Kernel:
         wait = lambda n: self.e(f"s_waitcnt vmcnt({min(63, n + (64 if first else 0))})")
         self.comment(f"---- chunk ({'first of a segment (' + str(first) + ')' if first else 'steady state'})")
         # step 0
-        wait(32 if two else 16)  # D0 of unit G+1 has landed
+        wait(24 if two else 8)  # D0 of unit G+1 has landed
         self.transform("D0")
         self.u_offset(self.sr("UoffM"), self.sr("KgM"), self.sr("Cm"), True)
         wait(16 if two else 0)  # U0 of this unit has landed
@@ -698,7 +702,7 @@ class Kernel:
         self.mfma_step(1, first, lambda p: self.load_patch("D0", p))
         # step 2
         if two:
-            self.e("s_waitcnt vmcnt(%d)" % (63 if first else 32))  # D1 of unit G+1 has landed
+            self.e("s_waitcnt vmcnt(%d)" % (63 if first else 24))  # D1 of unit G+1 has landed
             self.transform("D1")
         self.u_offset(self.sr("UoffQ"), self.sr("KgQ"), self.sr("Cq"), False)
         self.e("s_waitcnt vmcnt(16)")  # U1 (step 0) has landed; only D0 (step 1) is younger
@@ -1046,8 +1050,8 @@ class Kernel:
         e(f"v_add_u32 {self.vr('Off', 1)}, {self.sr('ColStep')}, {self.vr('Off', 0)}")
         e(f"v_add_u32 {self.vr('Off', 2)}, {self.sr('RowStep')}, {self.vr('Off', 0)}")
         e(f"v_add_u32 {self.vr('Off', 3)}, {self.sr('ColStep')}, {self.vr('Off', 2)}")
-        e(f"v_lshlrev_b32 {self.vr('Lane8')}, 3, {self.vr('Lane')}")
-        e(f"v_add_u32 {self.vr('Lane8b')}, 0x1000, {self.vr('Lane8')}")
+        e(f"v_lshlrev_b32 {self.vr('LaneU')}, 4, {self.vr('Lane')}")
+        e(f"v_add_u32 {self.vr('LaneUb')}, 0x1000, {self.vr('LaneU')}")
         # LDS: V[cw][buf][step][p][lane] floats.  Lds = read buffer, LdsWr = write buffer + this
         # wave's first owned step; the prologue writes buffer 0, which the swap in end_of_chunk
         # then makes the read buffer.

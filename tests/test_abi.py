@@ -132,6 +132,6 @@ def test_unswizzle_is_a_permutation(ocn):
     a = np.arange(C * 16 * K, dtype=np.float32)
     b = ocn.unswizzle_ww(a, C, K)
     assert sorted(b.ravel().tolist()) == a.tolist()
-    # element (kg=1, q=1, p=3, h=1, k32=5, s=1) is c = 4+2+1 = 7, k = 37
-    idx = ((((1 * (C // 4) + 1) * 16 + 3) * 2 + 1) * 32 + 5) * 2 + 1
+    # element (kg=1, q=1, p/2=1, h=1, k32=5, p%2=1, s=1) is c = 4+2+1 = 7, k = 37, p = 3
+    idx = (((((1 * (C // 4) + 1) * 8 + 1) * 2 + 1) * 32 + 5) * 2 + 1) * 2 + 1
     assert b[7, 3, 37] == a[idx]
