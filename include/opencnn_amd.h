@@ -90,7 +90,7 @@ int opencnn_init(void);
  * arguments return hipErrorInvalidValue and launch nothing.  Supported: filt_h ==
  * filt_w == 3, m == 2, alpha == tile_size == 4, filt_c == in_c, out_* consistent with pad 1 /
  * stride 1, tiles_dim == opencnn_tiles_dim(in_w), in_h == in_w, every tensor below 2^31
- * elements.  in_n, in_c and filt_k are free: outside the reference's in_n % 32 == 0,
+ * elements and in_n*in_h*in_w below 2^28.  in_n, in_c and filt_k are free: outside the reference's in_n % 32 == 0,
  * filt_k % 64 == 0, in_c % 8 == 0 the groups are rounded up and the missing lanes, channels
  * and filters predicated (Ww must then hold opencnn_workspace_bytes(), which is more than the
  * reference's filt_k*filt_c*16 floats).

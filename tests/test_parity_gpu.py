@@ -796,6 +796,72 @@ def test_every_tile_order_computes_the_same_layer(ocn, oracle, torch_gpu, prec, 
         ocn.set_tile_order(8)
 
 
+def direct_conv_at(torch, xf, wd, points, C, H, W, N):
+    """fp64 direct convolution (pad 1) at the sampled (y, x, n) points, all filters: definition of
+    the layer, evaluated on the device by gathering the 3x3xC neighbourhood of every point."""
+    ys, xs, ns = points.unbind(1)
+    chan = torch.arange(C, device=xf.device, dtype=torch.int64)[None, :]
+    acc = torch.zeros(points.shape[0], wd.shape[3], device=xf.device, dtype=torch.float64)
+    for r in range(3):
+        for s in range(3):
+            yy, xx = ys + (r - 1), xs + (s - 1)
+            ok = (yy >= 0) & (yy < H) & (xx >= 0) & (xx < W)
+            at = ((chan * H + yy.clamp(0, H - 1)[:, None]) * W + xx.clamp(0, W - 1)[:, None]) * N + ns[:, None]
+            v = xf[at].double() * ok[:, None]
+            acc += v @ wd[:, r, s, :].double()
+    return acc
+
+
+@pytest.mark.parametrize("prec,N,C,H,K,kernel", [
+    ("f32", 512, 64, 224, 64, "wino_f32_asm_kw2"),     # 6.6 GB in, 6.6 GB out: 64-bit bases of the assembly kernels
+    ("f16", 512, 64, 224, 64, "wino_f16_asm_kw4"),
+    ("f32", 4096, 8, 224, 8, "wino_f32_fused"),        # five output rows pass 2^31 bytes: the assembly kernels step aside
+])
+def test_tensors_beyond_four_gigabytes(ocn, torch_gpu, prec, N, C, H, K, kernel):
+    # Largest sizes: both tensors close to the 2^31 - 1 elements the entry points accept (the
+    # reference indexes with int as well).  Too large for the CPU oracle, so: every output element
+    # written, nothing written outside, and 4000 random points plus the tensor's corners against
+    # the fp64 direct convolution evaluated at those points.
+    print(f"large tensors {prec} N={N} C={C} H={H} K={K}", flush=True)
+    torch = torch_gpu
+    dev = torch.device("cuda:0")
+    n_in, n_out, guard = C * H * H * N, K * H * H * N, 4096
+    assert 2 ** 30 < n_in < 2 ** 31 and 2 ** 30 < n_out < 2 ** 31
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(SEED_X)
+    xd = torch.empty(n_in, device=dev).uniform_(-1.0, 1.0, generator=gen)
+    w = ocn.synth_filter(K, C, seed=SEED_W)
+    wd = torch.from_numpy(w).to(dev)
+    ws = torch.empty(ocn.workspace_bytes(C, K) // 4, device=dev)
+    raw = torch.full((n_out + 2 * guard,), float("nan"), device=dev)
+    yd = raw[guard:guard + n_out]
+    try:
+        ocn.set_operand_precision({"f32": ocn.F32, "f16": ocn.F16}[prec])
+        ocn.filter_transform(wd, ws, K, C, ocn.FILTER_CRSK, ocn.WW_MFMA)
+        ocn.conv_forward_pretransformed(xd, ws, yd, N, C, H, H, K)
+        torch.cuda.synchronize()
+        assert ocn.last_kernel().startswith(kernel), ocn.last_kernel()
+        ocn.check_status()
+    finally:
+        ocn.set_operand_precision(ocn.F32)
+    assert bool(torch.isnan(raw[:guard]).all()) and bool(torch.isnan(raw[-guard:]).all()), "wrote outside the output"
+    assert not bool(torch.isnan(yd).any()), "an output element was never written"
+    pts = torch.stack([torch.randint(0, H, (4000,), generator=gen, device=dev),
+                       torch.randint(0, H, (4000,), generator=gen, device=dev),
+                       torch.randint(0, N, (4000,), generator=gen, device=dev)], dim=1)
+    corners = torch.tensor([[y, x, n] for y in (0, H - 1) for x in (0, H - 1) for n in (0, N - 1)], device=dev)
+    pts = torch.cat([corners, pts]).to(torch.int64)
+    want = direct_conv_at(torch, xd, wd, pts, C, H, H, N)
+    filt = torch.arange(K, device=dev, dtype=torch.int64)[None, :]
+    got = yd[((filt * H + pts[:, 0:1]) * H + pts[:, 1:2]) * N + pts[:, 2:3]].double()
+    rel = float((got - want).norm() / want.norm())
+    worst = float((got - want).abs().max() / want.abs().max())
+    bar = {"f32": (1e-5, 1e-4), "f16": (2e-3, 2e-2)}[prec]
+    assert rel <= bar[0] and worst <= bar[1], (rel, worst)
+    del xd, raw, yd
+    torch.cuda.empty_cache()
+
+
 def test_non_default_stream(ocn, oracle, torch_gpu):
     print("stream", flush=True)
     torch = torch_gpu
