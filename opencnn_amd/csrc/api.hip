@@ -631,14 +631,6 @@ int pack_columns(opencnn::ConvArgs* a, int cw, int kblocks, int chunks, CutTiles
   return 0;
 }
 
-// The assembly kernels address a lane's four outputs relative to the filter row of its wave's
-// first half through 32-bit offsets whose bit 31 marks "do not store": the other half's rows lie
-// four rows further, so five rows of the output must stay below 2^31 bytes.  (The patch slabs of
-// the fp16 / bf16 kernels hold four channels: the same bound covers them.)
-bool asm_offsets_fit(const opencnn::ConvArgs& a) {
-  return (long long)a.N * a.H * a.W * 4 * 5 <= kMaxElems;
-}
-
 int launch_asm(const opencnn::ConvArgs& a, int kw, int grid, bool ragged, bool packed, size_t lds_bytes,
                hipStream_t st) {
   DeviceState* ak = nullptr;
@@ -678,7 +670,7 @@ int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* lau
   // transform, multiply zeros and store nothing.  In the _ragged kernels the last chunk's missing
   // channels read as zeros (descriptor cut at the tensor's end) and meet zero rows of the padded
   // transformed filter; batch elements and filter rows that do not exist are masked per lane / row.
-  if (!asm_offsets_fit(a)) return 0;
+  if ((long long)a.N * a.H * a.W * 4 * 4 > kMaxElems) return 0;  // four-channel slab in bytes
   const int kblocks = (a.kgroups + 3) / 4, chunks = (int)(padded_c_h16(a.C) / 16);
   const long long nblocks = (long long)a.colgroups * kblocks;
   const long long usw_bytes = padded_c_h16(a.C) * 16 * padded_k_h16(a.K) * 2;
@@ -960,7 +952,7 @@ int launch_on_flag_set(opencnn::ConvArgs& a, const CallSettings& c) {
   };
   auto lds_bytes = [](int kw) { return (size_t)(4 / kw) * 2 * 4 * 16 * 64 * sizeof(float); };
 
-  if ((variant == OPENCNN_KERNEL_ASM || variant == OPENCNN_KERNEL_AUTO) && asm_offsets_fit(a)) {
+  if (variant == OPENCNN_KERNEL_ASM || variant == OPENCNN_KERNEL_AUTO) {
     // The assembly kernels take a last filter block with fewer than kw filter groups: a wave
     // without filters reads zeros past the end of Ww, multiplies them and stores no row (the
     // row masks of the _ragged kernels).  So: the kw that leaves the fewest such waves, 4 on a tie.
@@ -975,8 +967,8 @@ int launch_on_flag_set(opencnn::ConvArgs& a, const CallSettings& c) {
     if (int e = asm_grid(b, kw, (b.C + 7) / 8, kCutRanges, &grid)) return e;
     if (grid > 0)
       return launch_asm(b, kw, grid, ragged || b.kgroups % kw != 0, packed, lds_bytes(kw), st);
+    REQUIRE(variant != OPENCNN_KERNEL_ASM);
   }
-  REQUIRE(variant != OPENCNN_KERNEL_ASM);
   // The HIP C++ kernels: as many sharing waves as the (rounded-up) filter groups fill whole
   // workgroups of.
   int kw = 1;
