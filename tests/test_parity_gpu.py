@@ -581,6 +581,33 @@ def test_padded_channels_do_not_leak_non_finite_values(ocn, oracle, torch_gpu, p
         assert not bad.any()
 
 
+@pytest.mark.parametrize("prec", ["f32", "f16"])
+@pytest.mark.parametrize("N,C,H,K", [(64, 64, 56, 64), (64, 16, 12, 128), (20, 12, 9, 40), (32, 512, 7, 512)])
+def test_non_finite_inputs_spread_as_in_the_reference_arithmetic(ocn, oracle, torch_gpu, prec, N, C, H, K):
+    # An infinity or a NaN in the input reaches, through the 4x4 patches, whole 2x2 output tiles
+    # of every filter (inf - inf in the output transform), not only the 3x3 neighbourhood of a
+    # direct convolution: the restatement of the reference's arithmetic says where, and the
+    # kernels - tiles cut between workgroups and merged included - must agree element by element.
+    print(f"non-finite {prec} N={N} C={C} H={H} K={K}", flush=True)
+    x, w = make_tensors(ocn, N, C, H, H, K)
+    x[1, 0, 0, 0] = np.inf                     # a corner: part of one patch only
+    x[C - 1, H // 2, H // 2, N - 1] = -np.inf  # an odd / even boundary: up to four patches
+    x[C // 2, H - 1, 1, N // 2] = np.nan
+    quant = {"f32": 0, "f16": 1}[prec]
+    try:
+        ocn.set_operand_precision({"f32": ocn.F32, "f16": ocn.F16}[prec])
+        y = Runner(ocn, torch_gpu, x, w).split()
+    finally:
+        ocn.set_operand_precision(ocn.F32)
+    want = oracle.winograd_f32(x, w, quant)
+    assert np.isnan(want).any() and np.isinf(want).any()
+    assert np.array_equal(np.isnan(y), np.isnan(want))
+    assert np.array_equal(np.isposinf(y), np.isposinf(want)) and np.array_equal(np.isneginf(y), np.isneginf(want))
+    ok = np.isfinite(want)
+    rel, max_abs, max_ref = oracle.compare(np.where(ok, y, 0.0), np.where(ok, want, 0.0))
+    assert rel <= {"f32": REL_L2_WINOGRAD, "f16": 2e-5}[prec], rel
+
+
 # ---------------------------------------------------------------- layout shims
 
 @pytest.mark.parametrize("N,C,H,W,K", [(32, 8, 8, 8, 64), (64, 64, 56, 56, 64), (96, 1030, 5, 3, 33), (1, 1, 1, 1, 1),
