@@ -608,6 +608,30 @@ def test_non_finite_inputs_spread_as_in_the_reference_arithmetic(ocn, oracle, to
     assert rel <= {"f32": REL_L2_WINOGRAD, "f16": 2e-5}[prec], rel
 
 
+@pytest.mark.parametrize("variant", ["auto", "hip"])
+@pytest.mark.parametrize("N,C,H,K", [(32, 8, 8, 64), (64, 16, 12, 128), (32, 8, 6, 32)])
+def test_denormal_operands_and_products_are_not_flushed(ocn, oracle, torch_gpu, variant, N, C, H, K):
+    # The reference is compiled without flush-to-zero: denormal inputs, transformed filters,
+    # products and sums keep their bits.  Here: MFMA and vector ALU in the same mode (the
+    # kernels' descriptors ask for fp32 denormals), checked on tensors whose products lie below
+    # the smallest normal number.
+    print(f"denormals {variant} N={N} C={C} H={H} K={K}", flush=True)
+    rng = np.random.default_rng(7)
+    for sx, sw in ((1e-19, 1e-19), (1e-38, 1.0), (1.0, 1e-38), (1e-41, 1.0)):
+        x = (rng.uniform(-1, 1, (C, H, H, N)) * sx).astype(np.float32)
+        w = (rng.normal(size=(C, 3, 3, K)) * sw).astype(np.float32)
+        try:
+            ocn.set_kernel_variant(ocn.KERNEL_HIP if variant == "hip" else ocn.KERNEL_AUTO)
+            y = Runner(ocn, torch_gpu, x, w).split()
+        finally:
+            ocn.set_kernel_variant(ocn.KERNEL_AUTO)
+        want = oracle.winograd_f32(x, w)
+        assert np.abs(want).max() < 1e-36 and (want != 0).mean() > 0.99
+        assert (y != 0).mean() == (want != 0).mean()
+        rel, _, _ = oracle.compare(y, want)
+        assert rel <= REL_L2_WINOGRAD, (sx, sw, rel)
+
+
 # ---------------------------------------------------------------- layout shims
 
 @pytest.mark.parametrize("N,C,H,W,K", [(32, 8, 8, 8, 64), (64, 64, 56, 56, 64), (96, 1030, 5, 3, 33), (1, 1, 1, 1, 1),
