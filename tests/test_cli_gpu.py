@@ -29,7 +29,8 @@ def check_output(p, n, c, h, k, bound):
     fields = lines[0].split(",")
     assert len(fields) == 12
     ms, ref_tflops, tflops, pct, gbs, ms_main, ms_fx = map(float, fields[5:])
-    assert 0 < ms_main <= ms and 0 < ms_fx < ms and tflops > 0 and ref_tflops > 0 and pct > 0 and gbs > 0
+    # (the three times come from separate passes of a few calls each: no order between them is asserted)
+    assert ms > 0 and ms_main > 0 and ms_fx > 0 and tflops > 0 and ref_tflops > 0 and pct > 0 and gbs > 0
     m = re.search(r"\[max_error: (\S+)\]\[rel_l2: (\S+)\]\[non_finite: (\d+)\] of (\d+)", lines[-1])
     assert m, lines[-1]
     assert float(m.group(2)) <= bound and int(m.group(3)) == 0 and int(m.group(4)) == n * k * h * h
