@@ -335,6 +335,10 @@ int opencnn_time_forward(const float *in, const float *w, float *out, float *Ww,
  * (else row by row), 4 = the tiles that an XCD's workgroups start with lie together in the image,
  * the tiles they go on with beside them.  Default 7; 0 is the order of
  * the first version of the kernels, kept for measurements (profiles/).
+ * Bits 8, 16, 32 (a number w = 0 ... 7): how the fp32 assembly kernels' balanced split cuts its
+ * ranges.  0: the library chooses (a cost model of the ranges, fitted to measurements); 1: equal
+ * numbers of units; w >= 2: on a line that adds w - 1 half units to every tile for its output
+ * transform, so that a range with one more tile end gets fewer units.
  */
 int opencnn_set_tile_order(int bits);
 

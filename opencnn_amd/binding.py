@@ -204,7 +204,8 @@ def release_stream(stream) -> None:
 
 
 def set_tile_order(bits: int) -> None:
-    """Order of the tiles in the image (bits 1, 2, 4 of opencnn_set_tile_order; default 7)."""
+    """Order of the tiles in the image (bits 1, 2, 4 of opencnn_set_tile_order; default 7) and, in
+    bits 8 - 32, how the fp32 kernels' balanced split cuts its ranges (0: the library chooses)."""
     _check("opencnn_set_tile_order", lib().opencnn_set_tile_order(bits))
 
 

@@ -965,9 +965,56 @@ class Kernel:
         """The register that numbers this workgroup's range of units."""
         return self.sr("L")
 
+    def weighted_unit_range(self, owner, vt):
+        """The ranges cut on a weighted line: a tile counts 2 * Chunks for its units plus the cost
+        of its output transform in half units (vt = the sum; its magic number in (Mch, Sch);
+        UnitsQ / UnitsRem count weighted half units), so that a range with one more tile end gets
+        fewer units.  Weighted position v -> tile v / vt, chunk min((v % vt + 1) / 2, Chunks)."""
+        t, e = self.t, self.e
+        for which, dst in ((0, self.sr("Begin")), (1, t(5))):
+            if which:
+                e(f"s_add_u32 {t(0)}, {owner}, 1")
+            else:
+                e(f"s_mov_b32 {t(0)}, {owner}")
+            e(f"s_mul_i32 {t(1)}, {t(0)}, {self.sr('UnitsQ')}")
+            e(f"s_min_u32 {t(2)}, {t(0)}, {self.sr('UnitsRem')}")
+            e(f"s_add_u32 {t(1)}, {t(1)}, {t(2)}")          # weighted start of range `owner + which`
+            self.div(t(2), t(1), self.sr("Mch"), self.sr("Sch"))  # tile
+            e(f"s_mul_i32 {t(3)}, {t(2)}, {vt}")
+            e(f"s_sub_u32 {t(3)}, {t(1)}, {t(3)}")
+            e(f"s_add_u32 {t(3)}, {t(3)}, 1")
+            e(f"s_lshr_b32 {t(3)}, {t(3)}, 1")
+            e(f"s_min_u32 {t(3)}, {t(3)}, {self.sr('Chunks')}")  # chunk
+            if not which:
+                e(f"s_mov_b32 {self.sr('Tm')}, {t(2)}")
+                e(f"s_mov_b32 {self.sr('Cm')}, {t(3)}")
+            e(f"s_mul_i32 {t(2)}, {t(2)}, {self.sr('Chunks')}")
+            e(f"s_add_u32 {dst}, {t(2)}, {t(3)}")
+        e(f"s_sub_u32 {self.sr('Nunits')}, {t(5)}, {self.sr('Begin')}")
+        # a weighted start behind a tile's last chunk is the next tile's first unit
+        e(f"s_cmp_eq_u32 {self.sr('Cm')}, {self.sr('Chunks')}")
+        e(f"s_cselect_b32 {self.sr('Cm')}, 0, {self.sr('Cm')}")
+        e(f"s_addc_u32 {self.sr('Tm')}, {self.sr('Tm')}, 0")
+
     def unit_range(self, owner):
         """Begin, Nunits (units [Begin, Begin + Nunits): the first UnitsRem ranges take one more)
-        and the first unit's tile Tm and chunk Cm."""
+        and the first unit's tile Tm and chunk Cm.  Bits 8.. of the magic shift Sch (which 64-bit
+        shifts ignore), when not zero: the weight of an output transform in half units, and the
+        ranges are cut on the weighted line (weighted_unit_range)."""
+        t, e = self.t, self.e
+        plain, done = self.newlabel("plain_ranges"), self.newlabel("ranges_done")
+        e(f"s_lshr_b32 {self.sr('Kind')}, {self.sr('Sch')}, 8")  # Kind, SegEnd: free until the segment loop
+        e(f"s_cmp_eq_u32 {self.sr('Kind')}, 0")
+        e(f"s_cbranch_scc1 {plain}")
+        e(f"s_lshl_b32 {self.sr('SegEnd')}, {self.sr('Chunks')}, 1")
+        e(f"s_add_u32 {self.sr('SegEnd')}, {self.sr('SegEnd')}, {self.sr('Kind')}")
+        self.weighted_unit_range(owner, self.sr("SegEnd"))
+        e(f"s_branch {done}")
+        self.label(plain)
+        self.plain_unit_range(owner)
+        self.label(done)
+
+    def plain_unit_range(self, owner):
         t, e = self.t, self.e
         e(f"s_mul_i32 {self.sr('Begin')}, {owner}, {self.sr('UnitsQ')}")
         e(f"s_min_u32 {t(0)}, {owner}, {self.sr('UnitsRem')}")

@@ -241,6 +241,14 @@ class ScalarMachine:
                 r = x + y if "add" in op else x - y
                 self.scc = int(r > m or r < 0)
                 self.s[int(a[0][1:])] = r & m
+            elif op == "s_addc_u32":
+                r = self.val(a[1]) + self.val(a[2]) + self.scc
+                self.scc = int(r > m)
+                self.s[int(a[0][1:])] = r & m
+            elif op == "s_min_u32":
+                x, y = self.val(a[1]), self.val(a[2])
+                self.scc = int(x < y)
+                self.s[int(a[0][1:])] = min(x, y)
             elif op == "s_mul_i32":
                 self.s[int(a[0][1:])] = (self.val(a[1]) * self.val(a[2])) & m
             elif op == "s_mul_hi_u32":
@@ -354,3 +362,35 @@ def test_places_of_a_line_are_a_permutation_of_each_window(gen, gen_h16, family,
         assert sorted(window) == list(range(lo, nxt))
         begins = [t for t in range(lo, nxt) if (t + 1) * ranges // tiles > t * ranges // tiles]
         assert [placed[t] for t in begins] == list(range(lo, lo + len(begins)))
+
+
+@pytest.mark.parametrize("tiles,chunks,ranges,weight", [
+    (392, 8, 256, 2), (784, 8, 256, 3), (392, 16, 256, 1), (300, 8, 256, 4), (1176, 8, 256, 2), (256, 64, 256, 5),
+    (1000, 3, 128, 6), (257, 1, 256, 1), (12345, 32, 256, 2)])
+@pytest.mark.parametrize("kw", [2, 4])
+def test_weighted_ranges_cover_the_line_of_units(gen, kw, tiles, chunks, ranges, weight):
+    # fp32 kernels, ranges cut on the weighted line (a tile = 2 * chunks + weight half units): the
+    # emitted code, run for every range, must give ranges that follow each other without gap or
+    # overlap from unit 0 to the last unit, none empty, each starting at its (tile, chunk), and
+    # the ranges must be those of the closed form.
+    k = gen.Kernel(kw)
+    k.lines = []
+    k.weighted_unit_range(f"s{k.S['L']}", f"s{k.S['SegEnd']}")
+    code = list(k.lines)
+    assert not any("branch" in l or re.match(r"^\S+:$", l) for l in code)
+    vt = 2 * chunks + weight
+    total = tiles * vt
+    q, rem = divmod(total, ranges)
+    mg, sh = magic(vt)
+    pos = lambda v: (v // vt) * chunks + min((v % vt + 1) // 2, chunks)
+    at = 0
+    for L in range(ranges):
+        m = ScalarMachine()
+        m.s.update({k.S["L"]: L, k.S["SegEnd"]: vt, k.S["UnitsQ"]: q, k.S["UnitsRem"]: rem, k.S["Chunks"]: chunks,
+                    k.S["Mch"]: mg, k.S["Sch"]: sh | (weight << 8)})
+        m.run(code)
+        begin, n, tm, cm = (m.s[k.S[x]] for x in ("Begin", "Nunits", "Tm", "Cm"))
+        assert begin == at and n > 0 and cm < chunks and tm * chunks + cm == begin
+        assert begin == pos(L * q + min(L, rem)) and begin + n == pos((L + 1) * q + min(L + 1, rem))
+        at += n
+    assert at == tiles * chunks

@@ -844,7 +844,7 @@ def test_every_tile_order_computes_the_same_layer(ocn, oracle, torch_gpu, prec, 
         rel, _, _ = oracle.compare(y, results[7])
         assert rel <= 3e-6, f"order {order}: rel-L2 vs the default order {rel:.3e}"
     with pytest.raises(ocn.OpenCNNError):
-        ocn.set_tile_order(8)
+        ocn.set_tile_order(64)
 
 
 def direct_conv_at(torch, xf, wd, points, C, H, W, N):
@@ -911,6 +911,33 @@ def test_tensors_beyond_four_gigabytes(ocn, torch_gpu, prec, N, C, H, K, kernel)
     assert rel <= bar[0] and worst <= bar[1], (rel, worst)
     del xd, raw, yd
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("N,C,H,K,kernel", [(32, 64, 56, 64, "wino_f32_asm_kw2"), (48, 64, 56, 64, "wino_f32_asm_kw2_packed"),
+                                            (96, 256, 14, 256, "wino_f32_asm_kw4"), (96, 120, 28, 250, "wino_f32_asm_kw4_ragged")])
+def test_ranges_cut_on_a_weighted_line_compute_the_same_layer(ocn, oracle, torch_gpu, N, C, H, K, kernel):
+    # Balanced split of the fp32 assembly kernels: the library may cut the ranges on a line that
+    # weighs every tile's output transform (bits 8, 16, 32 of opencnn_set_tile_order force a
+    # weight: 1 + half units), which moves the cuts between workgroups and nothing else.
+    print(f"weighted ranges N={N} C={C} H={H} K={K}", flush=True)
+    x, w = make_tensors(ocn, N, C, H, H, K)
+    r = Runner(ocn, torch_gpu, x, w)
+    want = oracle.direct_conv_f64(x, w)
+    results = {}
+    try:
+        for forced in (0, 1, 2, 3, 4, 5, 6, 7):  # 0: the library's choice, 1: equal numbers of units
+            ocn.set_tile_order(7 | (forced << 3))
+            r.raw.fill_(float("nan"))
+            results[forced] = r.split()
+            assert ocn.last_kernel() == kernel and ocn.last_launch()[0] == 256
+    finally:
+        ocn.set_tile_order(7)
+    for forced, y in results.items():
+        assert not np.isnan(y).any(), f"weight {forced}: an output element was never written"
+        rel64, _, _ = oracle.compare(y, want)
+        assert rel64 <= 1e-5, f"weight {forced}: rel-L2 vs fp64 direct {rel64:.3e}"
+        rel, _, _ = oracle.compare(y, results[1])
+        assert rel <= 3e-6, f"weight {forced}: rel-L2 vs the equal split {rel:.3e}"
 
 
 def test_non_default_stream(ocn, oracle, torch_gpu):
