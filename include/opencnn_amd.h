@@ -338,7 +338,8 @@ int opencnn_time_forward(const float *in, const float *w, float *out, float *Ww,
  * Bits 8, 16, 32 (a number w = 0 ... 7): how the fp32 assembly kernels' balanced split cuts its
  * ranges.  0: the library chooses (a cost model of the ranges, fitted to measurements); 1: equal
  * numbers of units; w >= 2: on a line that adds w - 1 half units to every tile for its output
- * transform, so that a range with one more tile end gets fewer units.
+ * transform, so that a range with one more tile end gets fewer units (fp16 / bf16 kernels:
+ * w >= 1 replaces their fixed weight of 4 half units by w - 1).
  */
 int opencnn_set_tile_order(int bits);
 
