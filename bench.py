@@ -344,6 +344,9 @@ def main():
                          "accumulation in every case); the default is the reference's fp32")
     ap.add_argument("--settle-ms", type=float, default=300.0,
                     help="untimed back-to-back run before every measurement (0: measure from idle)")
+    ap.add_argument("--tile-order", type=int, default=None, metavar="BITS",
+                    help="opencnn_set_tile_order for this run (measurements of the tile order and of the "
+                         "weight of the ranges; default: the library's)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-layers", action="store_true", help="skip the per-layer table")
     ap.add_argument("--timeline", action="store_true",
@@ -370,6 +373,8 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     ocn.init()
+    if args.tile_order is not None:
+        ocn.set_tile_order(args.tile_order)
 
     if args.shape:
         args.workload = custom_layer(args.shape)
@@ -418,7 +423,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": layer.name, "N": layer.N, "C": layer.C, "H": layer.H,
                    "W": layer.H, "K": layer.K, "pad": 1, "stride": 1,
-                   "layout": "CHWN in, CRSK filters, KHWN out"},
+                   "layout": "CHWN in, CRSK filters, KHWN out",
+                   **({"tile_order": args.tile_order} if args.tile_order is not None else {})},
         "roofline": {
             "kernel": kernel_name + " (fused Winograd kernel), %d workgroups, flag set %d" % (grid, flag_set),
             "bound": "mfma",
