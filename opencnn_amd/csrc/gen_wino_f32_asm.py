@@ -30,7 +30,7 @@ inside a tile is the other workgroup's LAST segment (merges).  Three cursors wal
 
 Registers.  a[16p:16p+15] accumulator of Winograd position p (MFMA D layout: register r, lane
 (h, n) = filter row 8*(r/4) + 4h + r%4, batch element n).  U0 / U1: A operands of the two
-filter quads of a chunk, one dwordx2 per position.  D0 (and D1 when a wave owns two steps):
+filter quads of a chunk, one dwordx4 per pair of positions.  D0 (and D1 when a wave owns two steps):
 patches in flight.  VA / VB: B operands of the current / next MFMA step, read from LDS
 V[cw][buf][step][p][lane].  T / TO: transform temporaries.  VOFF: per-lane byte offsets of the
 16 patch elements (out of range = zero padding).  Off / Eff: the four per-lane store offsets
