@@ -9,7 +9,9 @@ Prints ONE JSON line: effective TFLOP/s (direct-convolution FLOPs 2*N*K*C*H*W*9 
 step), ms per layer, the roofline of the dominant kernel (fp32 MFMA, algorithmic
 flops 32*N*T*C*K per launch) and a CPU baseline (the fp64 direct convolution of the
 oracle on the host cores).  ``layers`` repeats the figures for every fp32 layer of the
-benchmark set; only ``config.workload`` is the timed K-step region.
+benchmark set, in the sustained state and (``from_idle_*``) under the reference's own protocol of
+one warm-up call and 100 timed calls from an idle device; only ``config.workload`` is the timed
+K-step region.
 """
 import argparse
 import json
@@ -345,8 +347,11 @@ def main():
     ap.add_argument("--settle-ms", type=float, default=300.0,
                     help="untimed back-to-back run before every measurement (0: measure from idle)")
     ap.add_argument("--tile-order", type=int, default=None, metavar="BITS",
-                    help="opencnn_set_tile_order for this run (measurements of the tile order and of the "
-                         "weight of the ranges; default: the library's)")
+                    help="opencnn_set_tile_order for this run (measurements of the tile order; default: "
+                         "the library's)")
+    ap.add_argument("--range-weight", type=int, default=None, metavar="HALF_UNITS",
+                    help="opencnn_set_range_weight for this run (weight of a tile end on the line the "
+                         "balanced split cuts its ranges from; default: the library's choice)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-layers", action="store_true", help="skip the per-layer table")
     ap.add_argument("--timeline", action="store_true",
@@ -375,6 +380,8 @@ def main():
     ocn.init()
     if args.tile_order is not None:
         ocn.set_tile_order(args.tile_order)
+    if args.range_weight is not None:
+        ocn.set_range_weight(args.range_weight)
 
     if args.shape:
         args.workload = custom_layer(args.shape)
@@ -424,7 +431,8 @@ def main():
         "config": {"workload": layer.name, "N": layer.N, "C": layer.C, "H": layer.H,
                    "W": layer.H, "K": layer.K, "pad": 1, "stride": 1,
                    "layout": "CHWN in, CRSK filters, KHWN out",
-                   **({"tile_order": args.tile_order} if args.tile_order is not None else {})},
+                   **({"tile_order": args.tile_order} if args.tile_order is not None else {}),
+                   **({"range_weight": args.range_weight} if args.range_weight is not None else {})},
         "roofline": {
             "kernel": kernel_name + " (fused Winograd kernel), %d workgroups, flag set %d" % (grid, flag_set),
             "bound": "mfma",
@@ -483,6 +491,9 @@ def main():
                     ocn.set_operand_precision(prec)
                     settle(torch, lay, args.settle_ms / 2)
                     tot, mn, fx = lay.kernel_times(20, 200)
+                    # the reference's own protocol on this layer, after the sustained figures: the
+                    # idle period it starts with puts the device back into its idle state
+                    idle_row = from_idle(torch, lay, m, peak)
                 finally:
                     ocn.set_operand_precision(ocn.F32)
                 extra = {}
@@ -495,6 +506,9 @@ def main():
                     "effective_tflops": d / (tot * 1e-3) / 1e12,
                     "mfma_tflops": m / (mn * 1e-3) / 1e12,
                     "mfma_frac_of_peak": m / (mn * 1e-3) / 1e12 / peak,
+                    "from_idle_ms_per_layer": idle_row["ms_per_step"],
+                    "from_idle_ms_fused_kernel": idle_row["ms_fused_kernel"],
+                    "from_idle_frac": idle_row["frac"],
                     "hbm_gbs_at_min_bytes": b / (tot * 1e-3) / 1e9,
                     "hbm_frac_of_peak_at_min_bytes": b / (tot * 1e-3) / 1e9 / PEAK_HBM_GBS,
                 })

@@ -8,11 +8,13 @@
  * kernel variant, balanced split, operand precision; opencnn_conv_forward_desc takes all of
  * them per call instead), the code objects of its assembly kernels (embedded in the library,
  * loaded once per device by opencnn_init or the first launch), 1.5 MB of static device memory
- * that the balanced split uses to hand tiles over between workgroups (48 sets of flags, zero
- * between launches; see opencnn_set_balanced_split), per device 200 bytes of pinned host memory
+ * that the balanced split uses to hand tiles over between workgroups (48 sets of flags and a spare, zero
+ * between launches; see opencnn_set_balanced_split), per device 452 bytes of pinned host memory
  * that the kernels report a failed hand-over in (opencnn_check_status) and 32 events, all made by
  * opencnn_init or the first launch on the device, and a host-side record of the transformed
  * filters it wrote (opencnn_filter_transform).
+ * Bench and test support (timing loop, timeline, tile order, wait limit, synthetic tensors) is
+ * declared in opencnn_amd_bench.h and exported by the same library.
  * All entry points return a hipError_t value as int (0 == hipSuccess); launches are
  * asynchronous on the selected stream, exactly like the reference, which returns
  * cudaGetLastError() right after its two launches
@@ -183,20 +185,36 @@ int opencnn_set_kernel_variant(int variant);
  *     launches run without the split (slower, same results; opencnn_last_launch tells).
  *     opencnn_release_stream(stream) waits for a stream and gives its set back at once, e.g.
  *     before the stream is destroyed.
- *   - launches recorded in a stream capture hold one of 16 further sets per (capture, stream)
- *     for the life of the process, since the graph may be replayed at any time on any stream;
- *     the seventeenth runs without the split.  Two executable graphs instantiated from one
- *     capture share its set and must not run at the same time.
+ *   - launches recorded in a stream capture hold one of 16 further sets per (capture, stream),
+ *     since the graph may be replayed at any time on any stream; only the caller knows when it
+ *     will never run again, so the set stays taken until opencnn_release_capture gives it back.
+ *     With all 16 taken, a captured launch runs without the split.  Two executable graphs
+ *     instantiated from one capture share its set and must not run at the same time.
  *   - a caller that wants neither limit passes flag storage of its own in
  *     opencnn_conv_desc.split_flags.
+ * Only launches that cut a tile between workgroups take a set; a layer whose tiles fill whole
+ * rounds of the compute units, or a kernel with one tile per workgroup, takes none.
+ *
+ * opencnn_release_capture(stream, flag_set): gives graph sets back once the graphs recorded with
+ * them will not run again and their last replay has completed (the caller vouches for both).
+ * flag_set >= 0: that set, as opencnn_last_launch reported it right after the captured call;
+ * flag_set < 0: every graph set whose launches were recorded on `stream` (on any stream when
+ * `stream` is NULL).  A service that captures a graph per shape calls it when it drops a graph.
+ *
+ * opencnn_unsplit_launches(): fused-kernel launches since the process started, on any thread and
+ * device, that would have cut tiles between workgroups and ran without the split because no flag
+ * set was free (slower, same results): a counter to watch where opencnn_last_launch is too local.
  */
 int opencnn_set_balanced_split(int enable);
 int opencnn_release_stream(void *stream);
+int opencnn_release_capture(void *stream, int flag_set);
+unsigned long long opencnn_unsplit_launches(void);
 
 /*
  * What this thread's last successful fused-kernel launch looked like: its number of workgroups
- * and its set of split-merge flags (0..47 a set of the library, 48 the caller's storage, -1
- * none: the split was off, not needed by any kernel that could run, or no set was free).
+ * and its set of split-merge flags (0..31 a set of a stream, 32..47 a set of a stream capture, 48
+ * the caller's storage, -1 none: the split was off, the launch cut no tile between workgroups,
+ * or no set was free).
  * Either pointer may be NULL.  For tests and logs; no counterpart in the reference.
  */
 int opencnn_last_launch(int *workgroups, int *flag_set);
@@ -212,15 +230,23 @@ int opencnn_last_launch(int *workgroups, int *flag_set);
  * flag sets of the current device at once: call it after synchronising (hipDeviceSynchronize
  * or the streams in use) to learn whether every launch so far, graph replays included, handed
  * its tiles over; it returns 0 or hipErrorLaunchFailure (and has then cleared the library's
- * flag sets; flag storage of a caller is the caller's to clear).
+ * flag sets).
+ * What a report covers: the host only sees the word at its next call, so launches that were
+ * queued on the same flags between the launch that gave up and the call that reports it (and
+ * replays of a graph until somebody asks) ran on flags that may be inconsistent: treat the output
+ * of EVERY launch on that stream or graph since the last clean check as invalid.
+ * Flag storage of a caller (opencnn_conv_desc.split_flags): every such buffer has a status word
+ * of its own (the library tells up to 64 buffers per device apart, by address;
+ * opencnn_release_split_flags(buffer) forgets one, e.g. before it is freed, and a 65th buffer is
+ * refused with hipErrorInvalidValue).  A give-up on buffer A is reported by the next call that
+ * brings A, and by opencnn_check_status, never by a call on another buffer; the library clears A
+ * (a kernel on that call's stream) when the next call brings it, not before: the memory is the
+ * caller's and may be gone.
  * The reference has no hand-over and no such state (one block per tile,
  * src/convolutionForward_32x64x8.cu:281).
- *
- * opencnn_set_wait_limit: the number of polls after which a wait gives up, for tests of this
- * path (0 restores the default of 2^20 polls).
  */
 int opencnn_check_status(void);
-int opencnn_set_wait_limit(unsigned polls);
+int opencnn_release_split_flags(const void *split_flags);
 
 /*
  * The reference's FX kernel as a call of its own (src/FX_m2.cu:51-91, launched at
@@ -272,7 +298,9 @@ int opencnn_conv_forward_pretransformed(const float *in, const float *Ww, float 
  *                      split_flags_bytes >= opencnn_split_flags_bytes() of device memory that the
  *                      caller zeroed once: the hand-over state of this call.  Calls that share
  *                      one such buffer must not overlap in time; calls with different buffers may,
- *                      on any number of streams and graphs.
+ *                      on any number of streams and graphs (see opencnn_check_status for how a
+ *                      failed hand-over on such a buffer is reported, and
+ *                      opencnn_release_split_flags).
  * A zero-initialised struct with struct_size, the pointers and the shape filled in selects
  * the defaults except for balanced_split, which a caller who wants the default sets to 1.
  */
@@ -316,44 +344,6 @@ int opencnn_conv_forward_static(const float *in, const float *w, float *out, int
 size_t opencnn_static_workspace_bytes(void);
 
 /*
- * Bench support, the library-side twin of the reference's timing loop
- * (src/openCNN_winograd.cu:426-444): `warmup` untimed calls, then `iters` back-to-back
- * calls bracketed by HIP events on the selected stream.  Writes mean milliseconds per
- * call of (a) filter transform + fused kernel, the quantity the reference reports,
- * (b) the fused kernel alone, (c) the filter transform alone.  Synchronises the stream.
- */
-int opencnn_time_forward(const float *in, const float *w, float *out, float *Ww,
-                         int in_n, int in_c, int in_h, int in_w, int filt_k, int warmup,
-                         int iters, float *ms_total, float *ms_main, float *ms_fx);
-
-/*
- * Bench support without a counterpart in the reference: the order in which the assembly kernels
- * walk through the tiles of the image, which decides how much of a tile's input patch is found in
- * the L2 of its XCD because a neighbouring tile has just read it.  Results do not depend on it.
- * Bits: 1 = neighbouring column tiles are neighbouring spatial tiles (else: the same spatial tile
- * of the next 32 batch elements), 2 = spatial tiles numbered in zigzag strips of two tile rows
- * (else row by row), 4 = the tiles that an XCD's workgroups start with lie together in the image,
- * the tiles they go on with beside them.  Default 7; 0 is the order of
- * the first version of the kernels, kept for measurements (profiles/).
- * Bits 8, 16, 32 (a number w = 0 ... 7): how the fp32 assembly kernels' balanced split cuts its
- * ranges.  0: the library chooses (a cost model of the ranges, fitted to measurements); 1: equal
- * numbers of units; w >= 2: on a line that adds w - 1 half units to every tile for its output
- * transform, so that a range with one more tile end gets fewer units (fp16 / bf16 kernels:
- * w >= 1 replaces their fixed weight of 4 half units by w - 1).
- */
-int opencnn_set_tile_order(int bits);
-
-/*
- * Bench support without a counterpart in the reference: a timeline of the assembly kernels.
- * While a buffer is set, the first wave of workgroup L of every later launch of those kernels
- * writes into device_buffer[L*64 ...]: [0] the number of stamps, [2], [3], ... the GPU's
- * 100 MHz realtime counter at kernel start, after the prologue, and before and after every output
- * transform (at most 62 stamps).  `bytes` is the size of the buffer; launches with more
- * workgroups than it holds records for do not record.  NULL / 0 turns it off (the default).
- */
-int opencnn_set_timeline_buffer(long long *device_buffer, size_t bytes);
-
-/*
  * Layout shims on the selected stream, device to device, src != dst: the reference's data_cpy
  * kernel (src/openCNN_winograd.cu:147-153) as used at :230 (NCHW input -> CHWN) and :235 (KCRS
  * filters -> CRSK), plus the way back for the result (KHWN -> NKHW, i.e. NCHW with K channels),
@@ -364,23 +354,6 @@ int opencnn_set_timeline_buffer(long long *device_buffer, size_t bytes);
 int opencnn_nchw_to_chwn(const float *src, float *dst, int n, int c, int h, int w);
 int opencnn_khwn_to_nkhw(const float *src, float *dst, int n, int k, int h, int w);
 int opencnn_kcrs_to_crsk(const float *src, float *dst, int k, int c);
-
-/* Layout of a synthetic input written by opencnn_synth_input. */
-enum { OPENCNN_INPUT_CHWN = 0, OPENCNN_INPUT_NCHW = 1 };
-/* Distribution of a synthetic tensor: uniform on [p0,p1) or normal(mean p0, std p1). */
-enum { OPENCNN_DIST_UNIFORM = 0, OPENCNN_DIST_NORMAL = 1 };
-
-/*
- * Seeded synthetic tensors in HOST memory (no GPU involved).  They stand in for the
- * reference's unseeded curand fills and data_cpy transposes
- * (src/openCNN_winograd.cu:127-153,221-238): element values depend only on
- * (seed, logical NCHW / KCRS coordinate), so both layouts of a tensor hold the same
- * numbers.  Return 0, or 1 on a bad argument.
- */
-int opencnn_synth_input(float *dst, int n, int c, int h, int w, int layout,
-                        unsigned long long seed, int dist, double p0, double p1);
-int opencnn_synth_filter(float *dst, int k, int c, int layout, unsigned long long seed,
-                         int dist, double p0, double p1);
 
 /* Name of the last failing check in this thread ("" if none): a short static string. */
 const char *opencnn_last_error(void);

@@ -25,7 +25,8 @@ F32, F16, BF16 = 0, 1, 2
 
 _c_int, _c_float_p, _c_void_p = ctypes.c_int, ctypes.POINTER(ctypes.c_float), ctypes.c_void_p
 
-# name -> (restype, argtypes); one entry per declaration in include/opencnn_amd.h
+# name -> (restype, argtypes); one entry per declaration in include/opencnn_amd.h and
+# include/opencnn_amd_bench.h
 EXPORTED_SYMBOLS = {
     "opencnn_init": (_c_int, []),
     "convolutionForward": (
@@ -78,6 +79,10 @@ EXPORTED_SYMBOLS = {
     "opencnn_release_stream": (_c_int, [_c_void_p]),
     "opencnn_set_wait_limit": (_c_int, [ctypes.c_uint]),
     "opencnn_set_tile_order": (_c_int, [_c_int]),
+    "opencnn_set_range_weight": (_c_int, [_c_int]),
+    "opencnn_release_capture": (_c_int, [_c_void_p, _c_int]),
+    "opencnn_release_split_flags": (_c_int, [_c_void_p]),
+    "opencnn_unsplit_launches": (ctypes.c_ulonglong, []),
     "opencnn_forget_workspace": (_c_int, [_c_void_p]),
     "opencnn_conv_forward_desc": (_c_int, [_c_void_p]),
     "opencnn_split_flags_bytes": (ctypes.c_size_t, []),
@@ -204,9 +209,32 @@ def release_stream(stream) -> None:
 
 
 def set_tile_order(bits: int) -> None:
-    """Order of the tiles in the image (bits 1, 2, 4 of opencnn_set_tile_order; default 7) and, in
-    bits 8 - 32, how the fp32 kernels' balanced split cuts its ranges (0: the library chooses)."""
+    """Order of the tiles in the image for this thread's later launches (bits 1, 2, 4 of
+    opencnn_set_tile_order; default 7)."""
     _check("opencnn_set_tile_order", lib().opencnn_set_tile_order(bits))
+
+
+def set_range_weight(half_units: int) -> None:
+    """How this thread's later launches cut the ranges of the balanced split: -1 the library
+    chooses, 0 equal numbers of units, 1 ... 6 half units per tile end."""
+    _check("opencnn_set_range_weight", lib().opencnn_set_range_weight(half_units))
+
+
+def release_capture(stream=None, flag_set: int = -1) -> None:
+    """Give graph flag sets back: the set `flag_set`, or every set recorded on `stream` (None: on
+    any stream).  The graphs recorded with them must not run again."""
+    handle = 0 if stream is None else getattr(stream, "cuda_stream", stream)
+    _check("opencnn_release_capture", lib().opencnn_release_capture(handle, flag_set))
+
+
+def release_split_flags(split_flags) -> None:
+    """Forget a caller-owned flag buffer (its status word is free for another buffer)."""
+    _check("opencnn_release_split_flags", lib().opencnn_release_split_flags(_ptr(split_flags)))
+
+
+def unsplit_launches() -> int:
+    """Launches so far that wanted to cut tiles between workgroups and found no flag set free."""
+    return lib().opencnn_unsplit_launches()
 
 
 def set_wait_limit(polls: int) -> None:

@@ -2,6 +2,7 @@
 // Host-side counterpart of the reference's dispatcher and launcher
 // (src/openCNN_winograd.cu:204-219, src/convolutionForward_32x64x8.cu:264-284).
 #include "../../include/opencnn_amd.h"
+#include "../../include/opencnn_amd_bench.h"
 
 #include <hip/hip_runtime.h>
 
@@ -22,15 +23,22 @@ std::atomic<hipStream_t> g_stream{nullptr};
 std::atomic<int> g_variant{OPENCNN_KERNEL_AUTO};
 std::atomic<int> g_balance{1};
 std::atomic<int> g_precision{OPENCNN_F32};
-std::atomic<long long*> g_timeline{nullptr};
-std::atomic<size_t> g_timeline_bytes{0};
 std::atomic<bool> g_device_ready[64];  // set-up of device_state() done on that device
+// Bench and test support (include/opencnn_amd_bench.h): settings of the calling thread's own later
+// launches, so that one thread's measurement cannot change another thread's launch.
+thread_local long long* t_timeline = nullptr;
+thread_local size_t t_timeline_bytes = 0;
 // Polls after which a kernel's wait for a split-merge flag gives up (about a second).
 constexpr unsigned kDefaultWaitPolls = 1u << 20;
-std::atomic<unsigned> g_wait_polls{kDefaultWaitPolls};
+thread_local unsigned t_wait_polls = kDefaultWaitPolls;
 // Order of the tiles in the image (bits: 1 spatial tile fastest, 2 strips of two tile rows, 4 places
-// by starting time), see AsmLaunch; all on.  opencnn_set_tile_order is bench support.
-std::atomic<int> g_tile_order{7};
+// by starting time), see AsmLaunch; all on.
+thread_local int t_tile_order = 7;
+// Weight of a tile end on the line the ranges of the balanced split are cut from, in half units;
+// -1: the library chooses.
+thread_local int t_range_weight = -1;
+// Fused-kernel launches that wanted to cut tiles between workgroups and found no flag set free.
+std::atomic<unsigned long long> g_unsplit_launches{0};
 
 // The settings of one call: what the opencnn_set_* calls select for the entry points that take no
 // descriptor, or the fields of an opencnn_conv_desc.
@@ -91,8 +99,18 @@ struct FlagSetOwner {
   bool idle_recorded = false;
 };
 
-// Index of the status word of flag storage that a caller passed in a descriptor.
+// What opencnn_last_launch reports for flag storage that a caller passed in a descriptor.
 constexpr int kCallerSet = opencnn::kSyncSets;
+// Flag storage of callers that the library tells apart: each has a status word of its own.
+constexpr int kCallerSlots = 64;
+// Status words: one per flag set of the library, one per caller slot, one that nothing reads (for
+// launches that hand nothing over).
+constexpr int kStatusWords = opencnn::kSyncSets + kCallerSlots + 1;
+constexpr int kNoStatus = kStatusWords - 1;
+
+struct CallerFlags {
+  const unsigned* ptr = nullptr;
+};
 
 struct DeviceState {
   hipModule_t module = nullptr, module_h16 = nullptr;
@@ -102,12 +120,13 @@ struct DeviceState {
   hipFunction_t f16_kw4_packed = nullptr, bf16_kw4_packed = nullptr;
   unsigned* split_sync = nullptr;  // device address of g_split_sync (all sets) on this device
   float* scratch = nullptr;        // device address of `scratch` on this device
-  // One status word per flag set plus one for callers' own flag storage, in pinned host memory
-  // that the GPU writes directly: a wave that gives up waiting for a flag stores 1 there, and
-  // the host sees it at its next call without a copy or a synchronisation.
+  // Status words (kStatusWords) in pinned host memory that the GPU writes directly: a wave that
+  // gives up waiting for a flag stores 1 there, and the host sees it at its next call without a
+  // copy or a synchronisation.
   volatile unsigned* status_host = nullptr;
   unsigned* status_dev = nullptr;
   FlagSetOwner owners[opencnn::kSyncSets];
+  CallerFlags callers[kCallerSlots];
   unsigned long long clock = 0;
   bool pressure = false;  // more streams have launched than there are eager sets
   std::mutex flag_mu;
@@ -146,8 +165,8 @@ int device_state(DeviceState** out) {
       return (int)e;
     void* host = nullptr;
     void* dev_view = nullptr;
-    if ((e = hipHostMalloc(&host, (kCallerSet + 1) * sizeof(unsigned), hipHostMallocMapped)) != hipSuccess) return (int)e;
-    std::memset(host, 0, (kCallerSet + 1) * sizeof(unsigned));
+    if ((e = hipHostMalloc(&host, kStatusWords * sizeof(unsigned), hipHostMallocMapped)) != hipSuccess) return (int)e;
+    std::memset(host, 0, kStatusWords * sizeof(unsigned));
     if ((e = hipHostGetDevicePointer(&dev_view, host, 0)) != hipSuccess) return (int)e;
     k.status_host = static_cast<volatile unsigned*>(host);
     k.status_dev = static_cast<unsigned*>(dev_view);
@@ -183,7 +202,8 @@ DeviceState* device_state_if_ready() {
 //     one.  opencnn_release_stream returns a set explicitly;
 //   * launches recorded during a stream capture may be replayed on any stream at any time, so
 //     they never share a set with direct launches: every (capture, stream) pair holds one of the
-//     kGraphSets graph sets for the life of the process.
+//     kGraphSets graph sets until the caller gives it back (release_graph_sets): only the caller
+//     knows when a graph will never run again.
 // *set stays -1 when none is free: that launch then does without the split.  A set that is handed
 // out is marked as having a call in flight until flag_set_launched().
 int flag_set_for(DeviceState* ds, hipStream_t st, int* set) {
@@ -255,6 +275,55 @@ int release_flag_set(DeviceState* ds, hipStream_t st) {
     }
   }
   return 0;
+}
+
+// Gives graph sets back: the set `flag_set`, or (flag_set < 0) every set whose launches were
+// recorded on `st` (any stream when null).  The caller vouches that the graphs recorded with them
+// will not run again and that their last replay has completed.
+int release_graph_sets(DeviceState* ds, hipStream_t st, int flag_set) {
+  std::lock_guard<std::mutex> lock(ds->flag_mu);
+  for (int i = opencnn::kEagerSets; i < opencnn::kSyncSets; ++i) {
+    FlagSetOwner& o = ds->owners[i];
+    if (!o.used || o.calls_in_flight != 0) continue;
+    if (flag_set >= 0 ? i != flag_set : (st != nullptr && o.stream != st)) continue;
+    if (ds->status_host[i] != 0) {
+      // a replay gave up a hand-over and nobody asked: the next owner starts from clean flags
+      const hipError_t e = hipMemset(ds->split_sync + (size_t)i * opencnn::kSyncWords, 0,
+                                     opencnn::kSyncWords * sizeof(unsigned));
+      if (e != hipSuccess) return (int)e;
+      ds->status_host[i] = 0;
+    }
+    o.used = false;
+  }
+  return 0;
+}
+
+// The status word of flag storage that a caller owns: the slot that holds its address, else a free
+// one.  *slot stays -1 when the table is full.
+void caller_slot_for(DeviceState* ds, const unsigned* flags, int* slot) {
+  *slot = -1;
+  std::lock_guard<std::mutex> lock(ds->flag_mu);
+  int spare = -1;
+  for (int i = 0; i < kCallerSlots; ++i) {
+    if (ds->callers[i].ptr == flags) {
+      *slot = i;
+      return;
+    }
+    if (ds->callers[i].ptr == nullptr && spare < 0) spare = i;
+  }
+  if (spare < 0) return;
+  ds->callers[spare].ptr = flags;
+  ds->status_host[opencnn::kSyncSets + spare] = 0;
+  *slot = spare;
+}
+
+void release_caller_slot(DeviceState* ds, const unsigned* flags) {
+  std::lock_guard<std::mutex> lock(ds->flag_mu);
+  for (int i = 0; i < kCallerSlots; ++i)
+    if (ds->callers[i].ptr == flags) {
+      ds->callers[i].ptr = nullptr;
+      ds->status_host[opencnn::kSyncSets + i] = 0;
+    }
 }
 
 // Argument block of the assembly kernels (168 bytes, the layout gen_wino_f32_asm.py loads).
@@ -389,8 +458,15 @@ int launch_transpose(const float* src, float* dst, long long rows, long long col
   return (int)hipGetLastError();
 }
 
+// A launch is decided twice: first as a plan, under the assumption that hand-over flags are
+// available, to learn whether the kernel and grid it would choose cut any tile between workgroups;
+// only such a launch takes a flag set (or counts as a launch that found none).  Then for real.
+struct LaunchPlan {
+  bool cuts_tiles = false;
+};
+
 // fp16 / bf16 GEMM operands: 16-channel chunks, LDS kernel only; any N, C, K (RAGGED instantiations).
-int launch_h16(opencnn::ConvArgs a, int precision, hipStream_t st) {
+int launch_h16(opencnn::ConvArgs a, int precision, hipStream_t st, LaunchPlan* plan) {
   REQUIRE((long long)a.N * a.H * a.W * 4 * 4 <= kMaxElems);  // four-channel window in bytes
   const bool ragged = a.N % 32 != 0 || a.C % 16 != 0 || a.K % 64 != 0;
   a.kgroups = (int)(padded_k_h16(a.K) / 32);  // whole pairs of filter groups
@@ -411,6 +487,7 @@ int launch_h16(opencnn::ConvArgs a, int precision, hipStream_t st) {
       {{&opencnn::wino_h16_fused_lds<2, false, false>, &opencnn::wino_h16_fused_lds<2, false, true>},
        {&opencnn::wino_h16_fused_lds<2, true, false>, &opencnn::wino_h16_fused_lds<2, true, true>}}};
   const Kernel fn = kernels[kw == 2][bf][ragged];
+  if (plan != nullptr) return 0;  // a plain launch: one tile per workgroup
   if (kw == 2) {
     // 96 KB of LDS: above the 64 KB a kernel gets without asking (gfx950 has 160 KB per CU)
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn),
@@ -512,19 +589,19 @@ struct AsmLaunch {
   // Measured on the fp16 benchmark layer (N=128 C=K=256 14x14), fabric reads per launch: image
   // group fastest 124.6 MB, spatial tile fastest 93.2 MB (-3 % time); fp32 N=64 C=K=64 56x56
   // 155.5 -> 137.4 MB.
-  bool spatial_fastest = g_tile_order.load() & 1;
+  bool spatial_fastest = t_tile_order & 1;
   // Spatial tiles numbered in strips of two tile rows, zigzag, instead of row by row (fp32
   // N=64 C=K=64 56x56: 137.4 -> 129.3 MB, -0.5 % time).
-  bool strips = g_tile_order.load() & 2;
+  bool strips = t_tile_order & 2;
   // The tiles in work from the start get the first places of an XCD's window (Kernel.place;
   // 93.3 -> 82.4 MB on the fp16 benchmark layer).
-  bool tile_places = g_tile_order.load() & 4;
+  bool tile_places = t_tile_order & 4;
   // fp32 kernels: weight of a tile's output transform on the line the ranges are cut from, in half
   // units (0: equal numbers of units); travels in bits 8.. of the units' magic shift.
   int range_weight = 0;
 };
 
-int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmLaunch& l, hipStream_t st) {
+int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmLaunch& l, hipStream_t st, LaunchPlan* plan) {
   const int chunks = l.chunks, grid = l.grid;
   AsmKernArgs ka{};
   ka.x = a.x;
@@ -582,11 +659,16 @@ int launch_asm_kernel(const opencnn::ConvArgs& a, const AsmLaunch& l, hipStream_
   }
   ka.units_q = (int32_t)(total / ranges);
   ka.units_rem = (int32_t)(total % ranges);
+  if (plan != nullptr) {
+    // ranges of whole tiles (on the weighted line: whole weighted tiles) hand nothing over
+    plan->cuts_tiles = ka.units_rem != 0 || (uint32_t)ka.units_q % chunk_divisor != 0;
+    return 0;
+  }
   ka.usw_bytes = (int32_t)l.usw_bytes;
   ka.grid_per_xcd = grid % 8 == 0 ? grid / 8 : 0;  // 0: no XCD-aware block order
   ka.status = a.status;
   ka.wait_polls = a.spin_limit;
-  ka.timeline = (size_t)grid * 64 * sizeof(long long) <= g_timeline_bytes.load() ? g_timeline.load() : nullptr;
+  ka.timeline = (size_t)grid * 64 * sizeof(long long) <= t_timeline_bytes ? t_timeline : nullptr;
   magic_divisor(chunk_divisor, &ka.m_chunks, &ka.s_chunks);
   if (l.natural_order) ka.s_chunks |= 64;
   ka.s_chunks |= (uint32_t)range_weight << 8;
@@ -698,7 +780,7 @@ int choose_range_weight(int tiles, int chunks, int ranges) {
 }
 
 int launch_asm(const opencnn::ConvArgs& a, int kw, int grid, bool ragged, bool packed, size_t lds_bytes,
-               hipStream_t st) {
+               hipStream_t st, LaunchPlan* plan) {
   DeviceState* ak = nullptr;
   if (int e = device_state(&ak)) return e;
   AsmLaunch l;
@@ -720,11 +802,9 @@ int launch_asm(const opencnn::ConvArgs& a, int kw, int grid, bool ragged, bool p
   l.tile_split = a.colblocks;
   l.c_real_or_mode = a.C;
   // Ranges of the balanced split that are at least a tile long may be cut on a weighted line.
-  if (grid < a.nblocks && a.sync != nullptr) {
-    const int forced = (g_tile_order.load() >> 3) & 7;  // bench support: 1 + the weight
-    l.range_weight = forced > 0 ? forced - 1 : choose_range_weight(a.nblocks, l.chunks, grid);
-  }
-  return launch_asm_kernel(a, l, st);
+  if (grid < a.nblocks && a.sync != nullptr)
+    l.range_weight = t_range_weight >= 0 ? t_range_weight : choose_range_weight(a.nblocks, l.chunks, grid);
+  return launch_asm_kernel(a, l, st, plan);
 }
 
 // The hand-scheduled fp16 / bf16 kernels (gen_wino_h16_asm.py): 128-filter blocks, 16-channel
@@ -734,7 +814,7 @@ int launch_asm(const opencnn::ConvArgs& a, int kw, int grid, bool ragged, bool p
 // end on the weighted line of units counts 2, which also covers part of a cut tile's hand-over.
 constexpr int kEpilogueHalfUnits = 4;  // (weights 0 ... 6 on eleven layers: 4 is 0.3 % faster than 3 on average, -3 % at best)
 
-int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* launched) {
+int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* launched, LaunchPlan* plan) {
   *launched = false;
   bool packed = false;
   if (int e = pack_columns(&a, 1, (a.kgroups + 3) / 4, (int)(padded_c_h16(a.C) / 16), kCutPieces, &packed)) return e;
@@ -776,8 +856,7 @@ int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* lau
   l.lds_bytes = 2 * 16 * 2 * 4 * 32 * sizeof(unsigned);  // two buffers of V
   l.chunks = chunks;
   l.usw_bytes = usw_bytes;
-  const int forced_weight = (g_tile_order.load() >> 3) & 7;  // bench support: 1 + the weight
-  l.epilogue_half_units = cut_tiles ? 0 : (forced_weight > 0 ? forced_weight - 1 : kEpilogueHalfUnits);
+  l.epilogue_half_units = cut_tiles ? 0 : (t_range_weight >= 0 ? t_range_weight : kEpilogueHalfUnits);
   l.natural_order = cut_tiles;
   l.filters = a.K;
   // How the units are dealt.  While the whole 2-byte transformed filter leaves room in an XCD's
@@ -794,7 +873,7 @@ int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* lau
     l.tile_split = a.colblocks;
     l.c_real_or_mode = -a.C;
   }
-  const int e = launch_asm_kernel(a, l, st);
+  const int e = launch_asm_kernel(a, l, st, plan);
   *launched = e == 0;
   return e;
 }
@@ -802,8 +881,9 @@ int launch_h16_asm(opencnn::ConvArgs a, int precision, hipStream_t st, bool* lau
 // The HIP C++ kernels: register variant (kw == 1), LDS variant, and the LDS variant as one
 // continuous pipeline when the balanced split applies.
 int launch_hip(const opencnn::ConvArgs& a, int kw, bool ragged, bool allow_stream, size_t lds_bytes,
-               hipStream_t st) {
+               hipStream_t st, LaunchPlan* plan) {
   dim3 grid(((a.nblocks + 7) / 8) * 8), block(256);
+  if (plan != nullptr && (kw == 1 || ragged)) return 0;  // plain launches: one tile per workgroup
   if (kw == 1) {
     if (ragged)
       opencnn::wino_f32_fused<true><<<grid, block, 0, st>>>(a);
@@ -826,6 +906,10 @@ int launch_hip(const opencnn::ConvArgs& a, int kw, bool ragged, bool allow_strea
                         cus % 8 == 0 && cus <= opencnn::kMaxBalancedBlocks &&
                         (long long)a.nblocks * (a.C / 8) <= kMaxElems;
   if (balanced) grid = dim3(cus);
+  if (plan != nullptr) {
+    plan->cuts_tiles = balanced;
+    return 0;
+  }
   // The continuous pipeline pays off when a workgroup walks several tiles; for a single tile
   // per workgroup the plain LDS kernel has less scalar work per load.
   const bool stream = balanced && allow_stream;
@@ -919,38 +1003,62 @@ __global__ void zero_words(unsigned* p, int n) {
   if (i < n) p[i] = 0;
 }
 
+// Value of a caller buffer's status word after opencnn_check_status has reported it (a kernel stores 1).
+constexpr unsigned kReported = 2;
+
 const char* const kGaveUp =
     "an earlier launch gave up waiting for a partial tile (its output is invalid); the split-merge flags were cleared";
 
-// The flag set of this launch, and what an earlier launch may have left in its status word: a
-// wave that gave up a wait.  Then this call fails with hipErrorLaunchFailure and launches only
-// the kernel that clears the set (stream-ordered behind the launch that failed), so that the
-// call after it starts from clean flags.
-int prepare_split(DeviceState* ds, const CallSettings& c, opencnn::ConvArgs* a, int* taken) {
+// The flag set of a launch that cuts tiles between workgroups, and what an earlier launch may have
+// left in its status word: a wave that gave up a wait.  Then this call fails with
+// hipErrorLaunchFailure and launches only the kernel that clears the set (stream-ordered behind
+// the launch that failed), so that the call after it starts from clean flags.  A launch that hands
+// nothing over takes no set: it gets the spare one, which it never touches.
+int prepare_split(DeviceState* ds, const CallSettings& c, bool cuts_tiles, opencnn::ConvArgs* a, int* taken) {
   *taken = -1;
   a->sync = nullptr;
-  a->status = ds->status_dev + kCallerSet;
-  a->spin_limit = g_wait_polls.load();
+  a->status = ds->status_dev + kNoStatus;
+  a->spin_limit = t_wait_polls;
   t_last_flag_set = -1;
   if (!c.balance) return 0;
-  int set = -1;
+  if (!cuts_tiles) {
+    a->sync = ds->split_sync + (size_t)opencnn::kSyncSets * opencnn::kSyncWords;
+    return 0;
+  }
+  int set = -1, word = kNoStatus;
   if (c.caller_flags != nullptr) {
+    int slot = -1;
+    caller_slot_for(ds, c.caller_flags, &slot);
+    if (slot < 0)
+      return fail("too many flag buffers of callers in use (64): give one back with opencnn_release_split_flags");
     set = kCallerSet;
+    word = opencnn::kSyncSets + slot;
     a->sync = c.caller_flags;
   } else {
     if (int e = flag_set_for(ds, c.stream, &set)) return e;
-    if (set < 0) return 0;
+    if (set < 0) {
+      g_unsplit_launches.fetch_add(1);
+      return 0;
+    }
     *taken = set;
+    word = set;
     a->sync = ds->split_sync + (size_t)set * opencnn::kSyncWords;
   }
-  a->status = ds->status_dev + set;
-  if (ds->status_host[set] != 0) {
+  a->status = ds->status_dev + word;
+  const unsigned seen = ds->status_host[word];
+  if (seen != 0) {
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
     if (c.stream != nullptr) (void)hipStreamIsCapturing(c.stream, &capture);
     if (capture == hipStreamCaptureStatusNone) {  // (a capture would record the repair instead of running it)
       zero_words<<<(opencnn::kSyncWords + 255) / 256, 256, 0, c.stream>>>(a->sync, opencnn::kSyncWords);
       (void)hipGetLastError();
-      ds->status_host[set] = 0;
+      ds->status_host[word] = 0;
+      // kReported: opencnn_check_status has told the caller already; the buffer is clean again
+      // behind the kernel above, and this call goes ahead
+      if (seen == kReported) {
+        t_last_flag_set = set;
+        return 0;
+      }
     }
     flag_set_launched(ds, *taken, c.stream);
     *taken = -1;
@@ -961,7 +1069,7 @@ int prepare_split(DeviceState* ds, const CallSettings& c, opencnn::ConvArgs* a, 
   return 0;
 }
 
-int launch_on_flag_set(opencnn::ConvArgs& a, const CallSettings& c);
+int launch_on_flag_set(opencnn::ConvArgs& a, const CallSettings& c, LaunchPlan* plan);
 
 int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c, int in_h,
                 int in_w, int filt_k, const CallSettings& c) {
@@ -987,27 +1095,33 @@ int launch_main(const float* in, const float* Ww, float* out, int in_n, int in_c
   a.nblocks = a.colblocks = 0;
   DeviceState* ds = nullptr;
   if (int e = device_state(&ds)) return e;
+  LaunchPlan plan;
+  if (c.balance) {
+    opencnn::ConvArgs assumed = a;
+    assumed.sync = ds->split_sync;  // never dereferenced: it tells the choice that flags are to be had
+    if (int e = launch_on_flag_set(assumed, c, &plan)) return e;
+  }
   int set = -1;
-  if (int e = prepare_split(ds, c, &a, &set)) return e;
-  const int rc = launch_on_flag_set(a, c);
+  if (int e = prepare_split(ds, c, plan.cuts_tiles, &a, &set)) return e;
+  const int rc = launch_on_flag_set(a, c, nullptr);
   flag_set_launched(ds, set, c.stream);
   if (rc != 0) t_last_flag_set = -1;
   return rc;
 }
 
 // The fused kernel of a call whose split-merge state is in place.
-int launch_on_flag_set(opencnn::ConvArgs& a, const CallSettings& c) {
+int launch_on_flag_set(opencnn::ConvArgs& a, const CallSettings& c, LaunchPlan* plan) {
   const int in_n = a.N, in_c = a.C, filt_k = a.K, precision = c.precision;
   hipStream_t st = c.stream;
   if (precision != OPENCNN_F32) {
     const int v = c.variant;
     if (v == OPENCNN_KERNEL_ASM || v == OPENCNN_KERNEL_AUTO) {
       bool launched = false;
-      if (int e = launch_h16_asm(a, precision, st, &launched)) return e;
+      if (int e = launch_h16_asm(a, precision, st, &launched, plan)) return e;
       if (launched) return 0;
       REQUIRE(v != OPENCNN_KERNEL_ASM);
     }
-    return launch_h16(a, precision, st);
+    return launch_h16(a, precision, st, plan);
   }
 
   const bool ragged = ragged_shape(in_n, in_c, filt_k);
@@ -1039,7 +1153,7 @@ int launch_on_flag_set(opencnn::ConvArgs& a, const CallSettings& c) {
     int grid = 0;
     if (int e = asm_grid(b, kw, (b.C + 7) / 8, kCutRanges, &grid)) return e;
     if (grid > 0)
-      return launch_asm(b, kw, grid, ragged || b.kgroups % kw != 0, packed, lds_bytes(kw), st);
+      return launch_asm(b, kw, grid, ragged || b.kgroups % kw != 0, packed, lds_bytes(kw), st, plan);
     REQUIRE(variant != OPENCNN_KERNEL_ASM);
   }
   // The HIP C++ kernels: as many sharing waves as the (rounded-up) filter groups fill whole
@@ -1048,7 +1162,7 @@ int launch_on_flag_set(opencnn::ConvArgs& a, const CallSettings& c) {
   if (variant != OPENCNN_KERNEL_REGISTER) kw = a.kgroups % 4 == 0 ? 4 : (a.kgroups % 2 == 0 ? 2 : 1);
   if (variant == OPENCNN_KERNEL_LDS) REQUIRE(kw > 1);
   REQUIRE(tile_with(a, kw));
-  return launch_hip(a, kw, ragged, variant != OPENCNN_KERNEL_LDS, lds_bytes(kw), st);
+  return launch_hip(a, kw, ragged, variant != OPENCNN_KERNEL_LDS, lds_bytes(kw), st, plan);
 }
 
 bool valid_variant(int variant) {
@@ -1157,9 +1271,8 @@ int opencnn_set_operand_precision(int precision) {
 
 int opencnn_set_timeline_buffer(long long* device_buffer, size_t bytes) {
   REQUIRE((device_buffer == nullptr) == (bytes == 0));
-  g_timeline_bytes.store(0);
-  g_timeline.store(device_buffer);
-  g_timeline_bytes.store(bytes);
+  t_timeline = device_buffer;
+  t_timeline_bytes = bytes;
   return 0;
 }
 
@@ -1175,30 +1288,57 @@ int opencnn_release_stream(void* stream) {
 }
 
 int opencnn_set_tile_order(int bits) {
-  REQUIRE(bits >= 0 && bits <= 63);
-  g_tile_order.store(bits);
+  REQUIRE(bits >= 0 && bits <= 7);
+  t_tile_order = bits;
+  return 0;
+}
+
+int opencnn_set_range_weight(int half_units) {
+  REQUIRE(half_units >= -1 && half_units <= 6);
+  t_range_weight = half_units;
   return 0;
 }
 
 int opencnn_set_wait_limit(unsigned polls) {
-  g_wait_polls.store(polls == 0 ? kDefaultWaitPolls : polls);
+  t_wait_polls = polls == 0 ? kDefaultWaitPolls : polls;
   return 0;
 }
+
+int opencnn_release_capture(void* stream, int flag_set) {
+  REQUIRE(flag_set < 0 || (flag_set >= opencnn::kEagerSets && flag_set < opencnn::kSyncSets));
+  DeviceState* ds = device_state_if_ready();
+  if (ds == nullptr) return 0;
+  return release_graph_sets(ds, static_cast<hipStream_t>(stream), flag_set);
+}
+
+int opencnn_release_split_flags(const void* split_flags) {
+  DeviceState* ds = device_state_if_ready();
+  if (ds != nullptr) release_caller_slot(ds, static_cast<const unsigned*>(split_flags));
+  return 0;
+}
+
+unsigned long long opencnn_unsplit_launches(void) { return g_unsplit_launches.load(); }
 
 int opencnn_check_status(void) {
   DeviceState* ds = device_state_if_ready();
   if (ds == nullptr) return 0;  // nothing has been launched on this device
   bool gave_up = false;
-  for (int set = 0; set <= kCallerSet; ++set) {
+  for (int set = 0; set < opencnn::kSyncSets; ++set) {
     if (ds->status_host[set] == 0) continue;
     gave_up = true;
-    if (set < kCallerSet) {
-      // the caller has synchronised: nothing that uses the flags is running
-      const hipError_t e = hipMemset(ds->split_sync + (size_t)set * opencnn::kSyncWords, 0,
-                                     opencnn::kSyncWords * sizeof(unsigned));
-      if (e != hipSuccess) return (int)e;
-    }
+    // the caller has synchronised: nothing that uses the flags is running
+    const hipError_t e = hipMemset(ds->split_sync + (size_t)set * opencnn::kSyncWords, 0,
+                                   opencnn::kSyncWords * sizeof(unsigned));
+    if (e != hipSuccess) return (int)e;
     ds->status_host[set] = 0;
+  }
+  // Flag storage of callers: theirs to touch (it may be gone by now), so the word only changes to
+  // "reported", and the next call that brings the buffer clears it before it launches.
+  for (int slot = 0; slot < kCallerSlots; ++slot) {
+    volatile unsigned& word = ds->status_host[opencnn::kSyncSets + slot];
+    if (word == 0 || word == kReported) continue;
+    gave_up = true;
+    word = kReported;
   }
   if (!gave_up) return 0;
   t_last_error = kGaveUp;

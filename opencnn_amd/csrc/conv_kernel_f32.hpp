@@ -377,7 +377,8 @@ constexpr int kEagerSets = 32;  // streams that launch directly
 constexpr int kGraphSets = 16;  // launches recorded into HIP graphs
 constexpr int kSyncSets = kEagerSets + kGraphSets;
 constexpr int kSyncWords = kMaxBalancedBlocks * 4 * 2;
-static __device__ unsigned g_split_sync[kSyncSets * kSyncWords];
+// (one more set at the end for launches that cut no tile: they are given it and never touch it)
+static __device__ unsigned g_split_sync[(kSyncSets + 1) * kSyncWords];
 
 template <int KW, bool BALANCED, bool RAGGED = false>
 __global__ void __launch_bounds__(256) wino_f32_fused_lds(ConvArgs a) {

@@ -6,6 +6,7 @@
 // KCRS / CRSK views of a filter hold the same numbers, the relation the reference builds
 // with its data_cpy transposes (src/openCNN_winograd.cu:147-153,230,235).
 #include "../../include/opencnn_amd.h"
+#include "../../include/opencnn_amd_bench.h"
 
 #include <cmath>
 #include <cstdint>

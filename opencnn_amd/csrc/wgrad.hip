@@ -25,6 +25,7 @@
 #include <vector>
 
 #include "../../include/opencnn_amd.h"
+#include "../../include/opencnn_amd_bench.h"
 
 #define HIP_CALL(x)                                                                     \
   do {                                                                                  \

@@ -10,19 +10,24 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_functions():
-    text = open(os.path.join(ROOT, "include", "opencnn_amd.h")).read()
+def declared_functions(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b([A-Za-z_][A-Za-z0-9_]*)\s*\(", text)) - {"defined"})
 
 
 def test_header_symbols_exported(ocn):
-    names = declared_functions()
-    assert "convolutionForward" in names and "opencnn_filter_transform" in names
+    api, bench = declared_functions("opencnn_amd.h"), declared_functions("opencnn_amd_bench.h")
+    assert "convolutionForward" in api and "opencnn_filter_transform" in api
+    # bench and test support lives in its own header, and only there
+    assert set(bench) == {"opencnn_time_forward", "opencnn_set_tile_order", "opencnn_set_range_weight",
+                          "opencnn_set_wait_limit", "opencnn_set_timeline_buffer", "opencnn_synth_input",
+                          "opencnn_synth_filter"}
+    assert not set(api) & set(bench)
     handle = ctypes.CDLL(ocn.LIB_PATH)
-    for name in names:
-        assert hasattr(handle, name), f"{name} declared in include/opencnn_amd.h but not exported"
-    assert sorted(ocn.EXPORTED_SYMBOLS) == names  # the binding covers exactly the header
+    for name in api + bench:
+        assert hasattr(handle, name), f"{name} declared in include/ but not exported"
+    assert sorted(ocn.EXPORTED_SYMBOLS) == sorted(api + bench)  # the binding covers exactly the headers
 
 
 def test_tiles_dim_and_workspace(ocn, oracle):
@@ -102,6 +107,15 @@ def test_status_query_without_a_launch(ocn):
     assert ocn.lib().opencnn_set_wait_limit(0) == 0
     assert ocn.lib().opencnn_forget_workspace(0x1000) == 0
     assert ocn.last_launch() == (0, -1)
+    assert ocn.unsplit_launches() == 0
+    assert ocn.lib().opencnn_release_capture(None, -1) == 0
+    assert ocn.lib().opencnn_release_capture(None, 3) == 1     # not a graph set
+    assert ocn.lib().opencnn_release_capture(None, 48) == 1
+    assert ocn.lib().opencnn_release_split_flags(0x1000) == 0
+    for bad in (-2, 7):
+        assert ocn.lib().opencnn_set_range_weight(bad) == 1
+    assert ocn.lib().opencnn_set_range_weight(-1) == 0
+    assert ocn.lib().opencnn_set_tile_order(8) == 1 and ocn.lib().opencnn_set_tile_order(7) == 0
 
 
 def test_synth_layouts_agree(ocn):

@@ -194,6 +194,7 @@ def test_split_flags_owned_by_the_caller(ocn, torch_gpu, shape):
     assert ocn.last_launch()[1] == -1
     y = r.result()
     assert np.abs(y - want).max() <= 1e-4 * np.abs(want).max()
+    ocn.release_split_flags(flags)  # the library forgets the buffer before it is freed
 
 
 def test_more_streams_than_flag_sets(ocn, torch_gpu):
@@ -296,6 +297,165 @@ def test_replay_of_a_graph_overlaps_launches_on_its_capture_stream(ocn, torch_gp
         assert np.array_equal(rg.result(), want), f"replay {rep}"
         assert np.array_equal(re.result(), want), f"eager launches next to replay {rep}"
     ocn.check_status()
+
+
+def test_graph_flag_sets_are_given_back(ocn, torch_gpu):
+    # A launch recorded in a stream capture holds one of 16 graph sets until the caller gives it
+    # back: a service that captures a graph per shape would otherwise lose the balanced split from
+    # its 17th capture on.
+    print("graph flag sets", flush=True)
+    torch = torch_gpu
+    ocn.init()
+    N, C, H, W, K = CUT
+    x, w = make_tensors(ocn, N, C, H, W, K)
+    r = Runner(ocn, torch, x, w)
+    want = r.split()
+    grid = ocn.last_launch()[0]
+    s = torch.cuda.Stream()
+    ocn.release_capture(None)  # the graphs of earlier tests are gone
+
+    def capture():
+        g = torch.cuda.CUDAGraph()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(g, stream=s):
+            ocn.conv_forward_desc(r.xd, None, r.yd, r.ws, N, C, H, W, K, stream=s)
+        return g, ocn.last_launch()
+
+    def replay_is_right(g):
+        r.raw.fill_(float("nan"))
+        torch.cuda.synchronize()
+        g.replay()
+        return np.array_equal(r.result(), want)
+
+    # without a release the sets run out, and the counter says so
+    held = [capture() for _ in range(GRAPH_SETS)]
+    assert sorted(f for _, (_, f) in held) == list(range(EAGER_SETS, EAGER_SETS + GRAPH_SETS))
+    assert all(gr == grid for _, (gr, _) in held)
+    before = ocn.unsplit_launches()
+    g17, (grid17, set17) = capture()
+    assert set17 == -1 and grid17 != grid and ocn.unsplit_launches() == before + 1
+    y = None
+    r.raw.fill_(float("nan"))
+    torch.cuda.synchronize()
+    g17.replay()
+    y = r.result()  # without the split: another association of the channel sum
+    assert np.abs(y - want).max() <= 1e-4 * np.abs(want).max()
+    assert replay_is_right(held[3][0]) and replay_is_right(held[15][0])
+    # one set given back by number: the next capture gets exactly that one
+    del g17
+    torch.cuda.synchronize()
+    ocn.release_capture(None, held[5][1][1])
+    g, (gr, f) = capture()
+    assert (gr, f) == (grid, held[5][1][1]) and replay_is_right(g)
+    # all of this stream's sets given back, then twenty captures in a row, each released
+    del held, g
+    torch.cuda.synchronize()
+    ocn.release_capture(s)
+    before = ocn.unsplit_launches()
+    for i in range(20):
+        g, (gr, f) = capture()
+        assert gr == grid and f >= EAGER_SETS, f"capture {i} ran without the split"
+        assert replay_is_right(g), f"capture {i}"
+        del g
+        torch.cuda.synchronize()
+        ocn.release_capture(None, f)
+    assert ocn.unsplit_launches() == before
+    with pytest.raises(ocn.OpenCNNError):
+        ocn.release_capture(None, 3)  # a stream's set is not a graph set
+    ocn.check_status()
+
+
+def test_a_launch_that_cuts_no_tile_takes_no_flag_set(ocn, torch_gpu):
+    # 256 workgroup tiles on 256 compute units, one tile per workgroup, and the plumbing layer:
+    # nothing is handed over, so no set is taken (and none can run out).
+    print("no flag set", flush=True)
+    torch = torch_gpu
+    for shape in ((32, 16, 32, 16, 256), (32, 8, 8, 8, 64)):
+        N, C, H, W, K = shape
+        x, w = make_tensors(ocn, N, C, H, W, K)
+        r = Runner(ocn, torch, x, w)
+        before = ocn.unsplit_launches()
+        r.split()
+        assert ocn.last_launch()[1] == -1, shape
+        assert ocn.unsplit_launches() == before
+
+
+def test_caller_flag_buffers_report_on_their_own(ocn, torch_gpu):
+    # Every caller-owned flag buffer has its own status word: a hand-over that gave up on buffer A
+    # is reported by the next call that brings A (which also clears A), never by a call on B.
+    print("caller buffers, status", flush=True)
+    torch = torch_gpu
+    N, C, H, W, K = FEW
+    x, w = make_tensors(ocn, N, C, H, W, K)
+    r = Runner(ocn, torch, x, w)
+    want = r.split()
+    nwords = ocn.split_flags_bytes() // 4
+    A = torch.zeros(nwords, dtype=torch.int32, device="cuda")
+    B = torch.zeros(nwords, dtype=torch.int32, device="cuda")
+
+    def call(flags):
+        r.raw.fill_(float("nan"))
+        ocn.conv_forward_desc(r.xd, None, r.yd, r.ws, N, C, H, W, K, split_flags=flags)
+        return r.result()
+
+    assert np.array_equal(call(A), want) and np.array_equal(call(B), want)
+    gave_up = False
+    try:
+        ocn.set_wait_limit(1)
+        for _ in range(4):
+            if not np.array_equal(call(A), want):
+                gave_up = True
+                break
+    except ocn.OpenCNNError as e:
+        assert e.status == 719
+        pytest.fail("a give-up on A must be reported by the call after it, not by the one that gives up")
+    finally:
+        ocn.set_wait_limit(0)
+    if not gave_up:
+        ocn.release_split_flags(A)
+        ocn.release_split_flags(B)
+        pytest.skip("every hand-over found its partial tile at the first poll")
+    # B is clean and says nothing
+    assert np.array_equal(call(B), want)
+    # A reports once and is cleared by that call; then it works again
+    with pytest.raises(ocn.OpenCNNError) as e:
+        call(A)
+    assert e.value.status == 719 and "gave up" in e.value.detail
+    torch.cuda.synchronize()
+    assert int(A.abs().sum()) == 0
+    assert np.array_equal(call(A), want) and np.array_equal(call(B), want)
+    ocn.check_status()
+    ocn.release_split_flags(A)
+    ocn.release_split_flags(B)
+
+
+def test_caller_flag_buffers_beyond_the_table_are_refused(ocn, torch_gpu):
+    print("caller buffers, table", flush=True)
+    torch = torch_gpu
+    N, C, H, W, K = CUT
+    x, w = make_tensors(ocn, N, C, H, W, K)
+    r = Runner(ocn, torch, x, w)
+    want = r.split()
+    nwords = ocn.split_flags_bytes() // 4
+    pool = torch.zeros(65 * nwords, dtype=torch.int32, device="cuda")
+    bufs = [pool[i * nwords:(i + 1) * nwords] for i in range(65)]
+    try:
+        for b in bufs[:64]:
+            ocn.conv_forward_desc(r.xd, None, r.yd, r.ws, N, C, H, W, K, split_flags=b)
+        assert np.array_equal(r.result(), want)
+        r.raw.fill_(float("nan"))
+        with pytest.raises(ocn.OpenCNNError) as e:
+            ocn.conv_forward_desc(r.xd, None, r.yd, r.ws, N, C, H, W, K, split_flags=bufs[64])
+        assert e.value.status == 1 and "opencnn_release_split_flags" in e.value.detail
+        torch.cuda.synchronize()
+        assert torch.isnan(r.raw).all(), "a refused call must launch nothing"
+        ocn.release_split_flags(bufs[7])
+        ocn.conv_forward_desc(r.xd, None, r.yd, r.ws, N, C, H, W, K, split_flags=bufs[64])
+        assert np.array_equal(r.result(), want)
+    finally:
+        torch.cuda.synchronize()
+        for b in bufs:
+            ocn.release_split_flags(b)
 
 
 def test_a_wait_that_gives_up_is_reported(ocn, oracle, torch_gpu):

@@ -844,7 +844,7 @@ def test_every_tile_order_computes_the_same_layer(ocn, oracle, torch_gpu, prec, 
         rel, _, _ = oracle.compare(y, results[7])
         assert rel <= 3e-6, f"order {order}: rel-L2 vs the default order {rel:.3e}"
     with pytest.raises(ocn.OpenCNNError):
-        ocn.set_tile_order(64)
+        ocn.set_tile_order(8)
 
 
 def direct_conv_at(torch, xf, wd, points, C, H, W, N):
@@ -917,8 +917,8 @@ def test_tensors_beyond_four_gigabytes(ocn, torch_gpu, prec, N, C, H, K, kernel)
                                             (96, 256, 14, 256, "wino_f32_asm_kw4"), (96, 120, 28, 250, "wino_f32_asm_kw4_ragged")])
 def test_ranges_cut_on_a_weighted_line_compute_the_same_layer(ocn, oracle, torch_gpu, N, C, H, K, kernel):
     # Balanced split of the fp32 assembly kernels: the library may cut the ranges on a line that
-    # weighs every tile's output transform (bits 8, 16, 32 of opencnn_set_tile_order force a
-    # weight: 1 + half units), which moves the cuts between workgroups and nothing else.
+    # weighs every tile's output transform (opencnn_set_range_weight forces a weight in half
+    # units), which moves the cuts between workgroups and nothing else.
     print(f"weighted ranges N={N} C={C} H={H} K={K}", flush=True)
     x, w = make_tensors(ocn, N, C, H, H, K)
     r = Runner(ocn, torch_gpu, x, w)
@@ -926,12 +926,12 @@ def test_ranges_cut_on_a_weighted_line_compute_the_same_layer(ocn, oracle, torch
     results = {}
     try:
         for forced in (0, 1, 2, 3, 4, 5, 6, 7):  # 0: the library's choice, 1: equal numbers of units
-            ocn.set_tile_order(7 | (forced << 3))
+            ocn.set_range_weight(forced - 1)
             r.raw.fill_(float("nan"))
             results[forced] = r.split()
             assert ocn.last_kernel() == kernel and ocn.last_launch()[0] == 256
     finally:
-        ocn.set_tile_order(7)
+        ocn.set_range_weight(-1)
     for forced, y in results.items():
         assert not np.isnan(y).any(), f"weight {forced}: an output element was never written"
         rel64, _, _ = oracle.compare(y, want)
@@ -1073,8 +1073,10 @@ def test_call_replays_from_a_captured_graph(ocn, oracle, torch_gpu, N, C, H, K):
                 launch()
         # the captured launch is the eager one (same kernel, same grid) on a flag set of its own
         assert (ocn.last_kernel(), ocn.last_launch()[0]) == eager
-        assert ocn.last_launch()[1] >= 32, "the captured launch shares flags with direct launches"
-        if (N, C, H, K) != (32, 8, 8, 64):
+        if (N, C, H, K) == (32, 8, 8, 64):
+            assert ocn.last_launch()[1] == -1, "a launch that cuts no tile took a flag set"
+        else:
+            assert ocn.last_launch()[1] >= 32, "the captured launch shares flags with direct launches"
             assert ocn.last_kernel().startswith("wino_f32_asm") and ocn.last_launch()[0] > 64
         for rep in range(3):
             x2, w2 = ocn.synth_input(N, C, H, H, seed=100 + rep), ocn.synth_filter(K, C, seed=200 + rep)
