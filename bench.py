@@ -352,6 +352,9 @@ def main():
     ap.add_argument("--range-weight", type=int, default=None, metavar="HALF_UNITS",
                     help="opencnn_set_range_weight for this run (weight of a tile end on the line the "
                          "balanced split cuts its ranges from; default: the library's choice)")
+    ap.add_argument("--library", default=None, metavar="PATH",
+                    help="time another build of the library (make -C opencnn_amd/csrc diagnostic: "
+                         "kernels with parts of their work removed, WRONG RESULTS); the line says so")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-layers", action="store_true", help="skip the per-layer table")
     ap.add_argument("--timeline", action="store_true",
@@ -375,6 +378,8 @@ def main():
     import opencnn_amd as ocn
 
     ocn.load_library()  # raises if the HIP library is not built: there is no other path
+    if args.library:
+        ocn.use_library(args.library)
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     ocn.init()
@@ -465,6 +470,8 @@ def main():
             "ms_at_roof": roof_ms, "frac": roof_ms / ms_main,
             "mfma_frac_at_this_roof": fm / (roof_ms * 1e-3) / 1e12 / peak}
 
+    if args.library:
+        out["library"] = args.library + " (a diagnostic build: timing only, results are wrong)"
     if not args.no_cpu:
         from oracle import oracle
 

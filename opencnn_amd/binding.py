@@ -142,8 +142,16 @@ def load_library(path: str = LIB_PATH) -> ctypes.CDLL:
     return handle
 
 
+def use_library(path: str) -> ctypes.CDLL:
+    """Make another build of the same C ABI the library behind this module for the rest of the
+    process (the timing-only builds of `make -C opencnn_amd/csrc diagnostic`)."""
+    global _lib
+    _lib = load_library(path)
+    return _lib
+
+
 def lib() -> ctypes.CDLL:
-    return load_library()
+    return _lib if _lib is not None else load_library()
 
 
 def _ptr(buf) -> int:

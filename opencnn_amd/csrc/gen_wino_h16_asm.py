@@ -492,11 +492,34 @@ class KernelH16(Kernel):
         self.e(f"s_cmp_eq_u32 {self.sr('Cm')}, {self.sr('Chunks')}")
         self.e(f"s_cselect_b32 {self.sr('Cm')}, 0, {self.sr('Cm')}")
 
+    # Diagnostic builds (wrong results; make diagnostic): what is left of a unit.
+    #   "all"         the kernel
+    #   "loads_only"  the filter and patch loads with their waits: no MFMA, no transform, no LDS traffic
+    #   "no_units"    neither: scalar code, barrier, prologue, output transforms and hand-overs remain
+    KEEP = "all"
+
+    def kept(self, ops):
+        if self.KEEP == "all":
+            return ops
+        work = ("v_mfma", "v_sub_f32", "v_add_f32", "v_cvt_pk")
+        out = []
+        for op in ops:
+            if isinstance(op, str):
+                drop = op.split()[0].startswith(work)
+            elif isinstance(op, tuple):
+                drop = op[0] == "lds" or self.KEEP == "no_units"
+            else:
+                drop = op.counter == "lgkm" or self.KEEP == "no_units"
+            if not drop:
+                out.append(op)
+        return out
+
     def resolve(self, ops, first):
         """Emit the chunk with its s_waitcnt counts.  vmcnt: memory instructions issued after the
         awaited load, which sits behind its consumer in an earlier pass of the same sequence
         (cyclic count, saturated at the counter's 63: the wave then also waits for some younger
         loads).  lgkmcnt: LDS instructions issued after the awaited read, inside this chunk."""
+        ops = self.kept(ops)
         vm_pos = {op[2]: i for i, op in enumerate(ops) if isinstance(op, tuple) and op[0] == "vmem"}
         n_vm = sum(1 for op in ops if isinstance(op, tuple) and op[0] == "vmem")
         lds_pos = {op[2]: i for i, op in enumerate(ops) if isinstance(op, tuple) and op[0] == "lds" and op[2]}
@@ -510,7 +533,7 @@ class KernelH16(Kernel):
                 assert j > i, f"{op.tag} is awaited behind its reload"
                 after = sum(1 for o in ops[j + 1:] if isinstance(o, tuple) and o[0] == "vmem")
                 before = sum(1 for o in ops[:i] if isinstance(o, tuple) and o[0] == "vmem")
-                assert after + before < n_vm
+                assert after + before < n_vm or self.KEEP != "all"
                 # a filter load was issued by the previous chunk, a patch load by the one before
                 # that (same sequence of memory instructions in every chunk)
                 count = after + before + (0 if op.tag[0] == "U" else n_vm)
@@ -670,6 +693,10 @@ class KernelH16(Kernel):
 
 
 def main():
+    if len(sys.argv) == 3 and sys.argv[1] == "--keep" and sys.argv[2] in ("all", "loads_only", "no_units"):
+        KernelH16.KEEP = sys.argv[2]
+    elif len(sys.argv) > 1:
+        sys.exit("usage: gen_wino_h16_asm.py [--keep all|loads_only|no_units]")
     out = ['\t.amdgcn_target "amdgcn-amd-amdhsa--gfx950"', "\t.amdhsa_code_object_version 6"]
     kernels = [KernelH16(bf16, ragged, packed) for ragged, packed in ((False, False), (True, False), (True, True))
                for bf16 in (False, True)]
