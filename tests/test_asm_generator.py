@@ -202,6 +202,29 @@ def test_h16_flag_waits_are_bounded_and_report(gen_h16, bf16, ragged, packed):
     check_bounded_waits(k, "\n".join(k.lines))
 
 
+@pytest.mark.parametrize("keep", ["loads_only", "no_units"])
+def test_h16_diagnostic_builds_drop_what_they_say(gen_h16, keep, monkeypatch):
+    """gen_wino_h16_asm.py --keep (make diagnostic): timing-only kernels with the work of a unit taken
+    out.  The chunks lose their MFMAs, transform and LDS traffic (and, for no_units, their loads);
+    prologue, output transforms and hand-overs stay as they are."""
+    full = gen_h16.KernelH16(False)
+    full.body()
+    full_text = "\n".join(full.lines)
+    monkeypatch.setattr(gen_h16.KernelH16, "KEEP", keep)
+    k = gen_h16.KernelH16(False)
+    k.body()
+    text = "\n".join(k.lines)
+    assert "v_mfma" not in text
+    assert text.count("s_barrier") == full_text.count("s_barrier")
+    assert text.count("buffer_store_dword") == full_text.count("buffer_store_dword")
+    # the prologue's filter loads and LDS writes remain; the six chunk bodies' 16 + 32 loads only in loads_only
+    chunk_loads = 6 * 16 if keep == "loads_only" else 0
+    assert text.count("buffer_load_dwordx4") == 16 + chunk_loads
+    assert text.count("ds_read2st64_b32") == 0
+    assert text.count("ds_write2st64_b32") == 8
+    assert all(int(n) <= 63 for n in re.findall(r"vmcnt\((\d+)\)", text))
+
+
 @pytest.mark.skipif(not os.path.exists(CLANG), reason="ROCm LLVM assembler not installed")
 def test_h16_output_assembles_for_gfx950(tmp_path):
     src = tmp_path / "k.s"
