@@ -149,3 +149,20 @@ def test_unswizzle_is_a_permutation(ocn):
     # element (kg=1, q=1, p/2=1, h=1, k32=5, p%2=1, s=1) is c = 4+2+1 = 7, k = 37, p = 3
     idx = (((((1 * (C // 4) + 1) * 8 + 1) * 2 + 1) * 32 + 5) * 2 + 1) * 2 + 1
     assert b[7, 3, 37] == a[idx]
+
+
+def test_use_library_swaps_the_library_behind_the_module(ocn, tmp_path):
+    """bench.py --library: another build of the same C ABI becomes the library the wrappers call;
+    a path without a library is refused."""
+    import opencnn_amd.binding as binding
+
+    own = binding.lib()
+    try:
+        other = ocn.use_library(ocn.LIB_PATH)
+        assert binding.lib() is other
+        assert other.opencnn_tiles_dim(56) == 28
+        with pytest.raises(ImportError):
+            ocn.use_library(str(tmp_path / "libopencnn_amd_missing.so"))
+        assert binding.lib() is other
+    finally:
+        binding._lib = own
